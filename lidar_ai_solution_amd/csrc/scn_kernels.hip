@@ -1,0 +1,1398 @@
+// Hand-written gfx950 kernels of the SCN path and their launchers.
+//
+//   coordinate hash        atomicCAS open addressing over 64-bit {key,row} slots
+//   bitmap rank            occupancy bitmap + popcount scan: de-duplicates and orders keys
+//   rulebooks              output-stationary neighbour tables nbr[k][out] (+ pair compaction)
+//   gather-GEMM            MFMA 16x16x64 i8 / 16x16x32 f16, operands gathered straight into the
+//                          MFMA register layout, fused bias/requant/ReLU/residual epilogue
+//   elementwise            quantise / dequantise / pad, add(+relu)
+//   sparse -> dense        zero fill + strided scatter (covers the fused Transpose)
+//   voxelization           bitmap rank for voxel ids + atomicMin cascade for the kept points
+//
+// All kernels read row counts from device memory so that a forward pass never needs the host.
+#include "scn_kernels.hpp"
+
+#include <algorithm>
+#include <cstring>
+#include <type_traits>
+#include <vector>
+
+namespace scn {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+// --------------------------------------------------------------------------------------------
+// device helpers
+// --------------------------------------------------------------------------------------------
+// murmur3 finaliser evaluated in 64 bits (libraries/3DSparseConvolution/src/voxelization.cu:41-48)
+__host__ __device__ __forceinline__ uint64_t hash64(uint64_t k) {
+  k ^= k >> 16;
+  k *= 0x85ebca6bull;
+  k ^= k >> 13;
+  k *= 0xc2b2ae35ull;
+  k ^= k >> 16;
+  return k;
+}
+
+__device__ __forceinline__ void table_insert(uint64_t* slots, uint32_t mask, uint32_t key, uint32_t row) {
+  const uint64_t packed = ((uint64_t)key << 32) | row;
+  uint32_t slot = (uint32_t)hash64(key) & mask;
+  for (uint32_t probe = 0; probe <= mask; ++probe) {
+    unsigned long long prev = atomicCAS((unsigned long long*)&slots[slot], (unsigned long long)kEmptySlot,
+                                        (unsigned long long)packed);
+    if (prev == kEmptySlot) return;
+    if ((uint32_t)(prev >> 32) == key) {  // duplicate coordinate: the lowest row wins, deterministically
+      atomicMin((unsigned long long*)&slots[slot], (unsigned long long)packed);
+      return;
+    }
+    slot = (slot + 1) & mask;
+  }
+}
+
+__device__ __forceinline__ int32_t table_lookup(const uint64_t* __restrict__ slots, uint32_t mask, uint32_t key) {
+  uint32_t slot = (uint32_t)hash64(key) & mask;
+  for (uint32_t probe = 0; probe <= mask; ++probe) {
+    const uint64_t v = slots[slot];
+    if (v == kEmptySlot) return -1;
+    if ((uint32_t)(v >> 32) == key) return (int32_t)(uint32_t)v;
+    slot = (slot + 1) & mask;
+  }
+  return -1;
+}
+
+__device__ __forceinline__ uint32_t eff_n(const uint32_t* n_dev, uint32_t n_bound) {
+  if (n_dev == nullptr) return n_bound;
+  const uint32_t n = *n_dev;
+  return n < n_bound ? n : n_bound;
+}
+
+struct Int3 {
+  int v[3];
+};
+
+// Block-wide exclusive scan of one value per thread (blockDim.x multiple of 64, <= 1024).
+// Returns the exclusive prefix; *total receives the block sum.  scratch: >= 17 uint32 in LDS.
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t x, uint32_t* scratch, uint32_t* total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  uint32_t incl = x;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    uint32_t y = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += y;
+  }
+  __syncthreads();  // scratch may still be read from a previous call
+  if (lane == 63) scratch[wave] = incl;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    uint32_t s = 0;
+    for (int w = 0; w < nw; ++w) {
+      uint32_t t = scratch[w];
+      scratch[w] = s;
+      s += t;
+    }
+    scratch[16] = s;
+  }
+  __syncthreads();
+  *total = scratch[16];
+  return scratch[wave] + incl - x;
+}
+
+// --------------------------------------------------------------------------------------------
+// fill
+// --------------------------------------------------------------------------------------------
+__global__ void k_fill_u32(uint32_t* __restrict__ p, uint32_t value, size_t count) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  // 16-byte stores over the aligned body
+  const size_t n4 = count / 4;
+  uint4 v4 = make_uint4(value, value, value, value);
+  for (size_t j = i; j < n4; j += stride) reinterpret_cast<uint4*>(p)[j] = v4;
+  for (size_t j = n4 * 4 + i; j < count; j += stride) p[j] = value;
+}
+
+int fill_u32(void* p, uint32_t value, size_t count, hipStream_t stream) {
+  if (count == 0) return SCN_OK;
+  SCN_REQUIRE(((uintptr_t)p & 15) == 0, SCN_ERR_INVALID, "fill_u32: pointer not 16-byte aligned");
+  size_t blocks = (count / 4 + 255) / 256;
+  if (blocks < 1) blocks = 1;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(k_fill_u32, dim3((unsigned)blocks), dim3(256), 0, stream, (uint32_t*)p, value, count);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
+// --------------------------------------------------------------------------------------------
+// coordinate hash build / query
+// --------------------------------------------------------------------------------------------
+__device__ __forceinline__ bool coord_key(const int4 c, const Int3 g, uint32_t* key) {
+  if (c.x != 0 || c.y < 0 || c.y >= g.v[0] || c.z < 0 || c.z >= g.v[1] || c.w < 0 || c.w >= g.v[2]) return false;
+  *key = ((uint32_t)c.y * (uint32_t)g.v[1] + (uint32_t)c.z) * (uint32_t)g.v[2] + (uint32_t)c.w;
+  return true;
+}
+
+__global__ void k_hash_insert(uint64_t* slots, uint32_t mask, const int4* __restrict__ coords, uint32_t n_bound,
+                              const uint32_t* n_dev, Int3 grid, uint32_t* n_eff_out) {
+  const uint32_t n = eff_n(n_dev, n_bound);
+  const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r == 0 && n_eff_out) {
+    n_eff_out[0] = n;
+    n_eff_out[1] = n;
+  }
+  if (r >= n) return;
+  uint32_t key;
+  if (coord_key(coords[r], grid, &key)) table_insert(slots, mask, key, r);
+}
+
+__global__ void k_hash_query(const uint64_t* __restrict__ slots, uint32_t mask, const int4* __restrict__ coords,
+                             uint32_t n, Int3 grid, int32_t* rows) {
+  const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= n) return;
+  uint32_t key;
+  rows[r] = coord_key(coords[r], grid, &key) ? table_lookup(slots, mask, key) : -1;
+}
+
+size_t hash_capacity_for(uint32_t n) {
+  size_t cap = 1024;
+  while (cap < (size_t)n * 2) cap <<= 1;
+  return cap;
+}
+
+bool CoordTable::alloc_for(uint32_t max_rows) {
+  cap = hash_capacity_for(max_rows);
+  mask = (uint32_t)(cap - 1);
+  return buf.alloc(cap * sizeof(uint64_t));
+}
+
+static bool grid_fits_u32(const int g[3]) {
+  if (g[0] <= 0 || g[1] <= 0 || g[2] <= 0) return false;
+  const uint64_t vol = (uint64_t)g[0] * (uint64_t)g[1] * (uint64_t)g[2];
+  return vol < 0xFFFFFFFFull;
+}
+
+int hash_build(const CoordTable& t, const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3],
+               uint32_t* n_eff_out, hipStream_t stream) {
+  SCN_REQUIRE(t.cap >= hash_capacity_for(n), SCN_ERR_CAPACITY, "hash table capacity %zu too small for %u rows",
+              t.cap, n);
+  SCN_REQUIRE(grid_fits_u32(grid), SCN_ERR_UNSUPPORTED, "grid %dx%dx%d does not fit 32-bit keys", grid[0], grid[1],
+              grid[2]);
+  const_cast<CoordTable&>(t).mask = (uint32_t)(hash_capacity_for(n) - 1);
+  int rc = fill_u32(t.slots(), 0xFFFFFFFFu, ((size_t)t.mask + 1) * 2, stream);
+  if (rc) return rc;
+  Int3 g{{grid[0], grid[1], grid[2]}};
+  const uint32_t blocks = n ? ceil_div(n, 256) : 1;
+  hipLaunchKernelGGL(k_hash_insert, dim3(blocks), dim3(256), 0, stream, t.slots(), t.mask,
+                     (const int4*)idx, n, n_dev, g, n_eff_out);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
+int hash_query(const CoordTable& t, const int32_t* coords, uint32_t n, const int grid[3], int32_t* rows,
+               hipStream_t stream) {
+  if (n == 0) return SCN_OK;
+  Int3 g{{grid[0], grid[1], grid[2]}};
+  hipLaunchKernelGGL(k_hash_query, dim3(ceil_div(n, 256)), dim3(256), 0, stream, t.slots(), t.mask,
+                     (const int4*)coords, n, g, rows);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
+// --------------------------------------------------------------------------------------------
+// bitmap rank: block sums, scan of block sums, expansion
+// one block = 256 threads x 4 words = 1024 bitmap words
+// --------------------------------------------------------------------------------------------
+constexpr uint32_t kWordsPerBlock = 1024;
+
+__global__ __launch_bounds__(256) void k_bitmap_blocksum(const uint32_t* __restrict__ bitmap, uint32_t* blocksum) {
+  __shared__ uint32_t scratch[17];
+  const uint4 w = reinterpret_cast<const uint4*>(bitmap)[(size_t)blockIdx.x * 256 + threadIdx.x];
+  uint32_t c = __popc(w.x) + __popc(w.y) + __popc(w.z) + __popc(w.w);
+  uint32_t total;
+  (void)block_exclusive_scan(c, scratch, &total);
+  if (threadIdx.x == 0) blocksum[blockIdx.x] = total;
+}
+
+// Single block: in-place exclusive scan of `count` values; counters[1] = total, counters[0] = min(total, cap).
+__global__ __launch_bounds__(1024) void k_scan_blocksums(uint32_t* vals, uint32_t count, uint32_t* counters,
+                                                        uint32_t cap) {
+  __shared__ uint32_t scratch[17];
+  uint32_t carry = 0;
+  for (uint32_t base = 0; base < count; base += 1024) {
+    const uint32_t i = base + threadIdx.x;
+    const uint32_t x = i < count ? vals[i] : 0;
+    uint32_t total;
+    const uint32_t ex = block_exclusive_scan(x, scratch, &total);
+    if (i < count) vals[i] = carry + ex;
+    carry += total;
+  }
+  if (threadIdx.x == 0 && counters) {
+    counters[1] = carry;
+    counters[0] = carry < cap ? carry : cap;
+  }
+}
+
+// Expands the set bits in rank order.  Optional outputs: coordinate rows, a hash table of
+// {key -> rank}, and the per-word exclusive prefix (rank of the word's first bit).
+__global__ __launch_bounds__(256) void k_bitmap_expand(const uint32_t* __restrict__ bitmap,
+                                                       const uint32_t* __restrict__ blockoff, Int3 grid, uint32_t cap,
+                                                       int4* coords_out, uint64_t* slots, uint32_t mask,
+                                                       uint32_t* prefix_out) {
+  __shared__ uint32_t scratch[17];
+  const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const uint4 w4 = reinterpret_cast<const uint4*>(bitmap)[t];
+  const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
+  const uint32_t c = __popc(w[0]) + __popc(w[1]) + __popc(w[2]) + __popc(w[3]);
+  uint32_t total;
+  uint32_t rank = blockoff[blockIdx.x] + block_exclusive_scan(c, scratch, &total);
+  if (prefix_out) {
+    uint4 p;
+    p.x = rank;
+    p.y = p.x + __popc(w[0]);
+    p.z = p.y + __popc(w[1]);
+    p.w = p.z + __popc(w[2]);
+    reinterpret_cast<uint4*>(prefix_out)[t] = p;
+  }
+  if (c == 0 || coords_out == nullptr) return;
+  const uint32_t g12 = (uint32_t)grid.v[1] * (uint32_t)grid.v[2];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    uint32_t bits = w[j];
+    while (bits) {
+      const int b = __ffs(bits) - 1;
+      bits &= bits - 1;
+      if (rank < cap) {
+        const uint32_t key = (uint32_t)(t * 4 + j) * 32u + (uint32_t)b;
+        const uint32_t i0 = key / g12, rem = key - i0 * g12;
+        const uint32_t i1 = rem / (uint32_t)grid.v[2], i2 = rem - i1 * (uint32_t)grid.v[2];
+        coords_out[rank] = make_int4(0, (int)i0, (int)i1, (int)i2);
+        if (slots) table_insert(slots, mask, key, rank);
+      }
+      rank++;
+    }
+  }
+}
+
+static size_t bitmap_words_for(const int g[3]) {
+  const uint64_t vol = (uint64_t)g[0] * g[1] * g[2];
+  const uint64_t words = (vol + 31) / 32;
+  return (size_t)((words + kWordsPerBlock - 1) / kWordsPerBlock * kWordsPerBlock);
+}
+
+// --------------------------------------------------------------------------------------------
+// rulebooks
+// --------------------------------------------------------------------------------------------
+struct GeomDev {
+  int gi[3], go[3], ks[3], st[3], pd[3], dl[3];
+};
+
+static GeomDev to_dev(const ConvGeom& g) {
+  GeomDev d;
+  for (int a = 0; a < 3; ++a) {
+    d.gi[a] = g.grid_in[a];
+    d.go[a] = g.grid_out[a];
+    d.ks[a] = g.ks[a];
+    d.st[a] = g.stride[a];
+    d.pd[a] = g.pad[a];
+    d.dl[a] = g.dil[a];
+  }
+  return d;
+}
+
+// nbr[k][o] = row of the input at  o*stride - pad + k*dilation  (or -1).  grid.y = kernel offset.
+// Used for both kinds: submanifold passes stride 1 and pad = floor(K/2)*dilation.
+__global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_coords, const uint32_t* n_out_dev,
+                                                   uint32_t n_bound, GeomDev g, const uint64_t* __restrict__ slots,
+                                                   uint32_t mask, int32_t* nbr, uint32_t ld, int identity_center) {
+  const uint32_t n = eff_n(n_out_dev, n_bound);
+  const uint32_t o = blockIdx.x * 256 + threadIdx.x;
+  if (o >= n) return;
+  const int k = blockIdx.y;
+  const int k2 = k % g.ks[2], k1 = (k / g.ks[2]) % g.ks[1], k0 = k / (g.ks[2] * g.ks[1]);
+  const int4 c = out_coords[o];
+  int32_t res = -1;
+  if (identity_center && k0 == g.ks[0] / 2 && k1 == g.ks[1] / 2 && k2 == g.ks[2] / 2) {
+    res = (int32_t)o;
+  } else {
+    const int i0 = c.y * g.st[0] - g.pd[0] + k0 * g.dl[0];
+    const int i1 = c.z * g.st[1] - g.pd[1] + k1 * g.dl[1];
+    const int i2 = c.w * g.st[2] - g.pd[2] + k2 * g.dl[2];
+    if (c.x == 0 && i0 >= 0 && i0 < g.gi[0] && i1 >= 0 && i1 < g.gi[1] && i2 >= 0 && i2 < g.gi[2]) {
+      const uint32_t key = ((uint32_t)i0 * (uint32_t)g.gi[1] + (uint32_t)i1) * (uint32_t)g.gi[2] + (uint32_t)i2;
+      res = table_lookup(slots, mask, key);
+    }
+  }
+  nbr[(size_t)k * ld + o] = res;
+}
+
+// Marks every output cell reached by an input row through some kernel offset.  grid.y = offset.
+__global__ __launch_bounds__(256) void k_mark_outputs(const int4* __restrict__ in_coords, const uint32_t* n_dev,
+                                                      uint32_t n_bound, GeomDev g, uint32_t* bitmap) {
+  const uint32_t n = eff_n(n_dev, n_bound);
+  const uint32_t r = blockIdx.x * 256 + threadIdx.x;
+  if (r >= n) return;
+  const int k = blockIdx.y;
+  const int k2 = k % g.ks[2], k1 = (k / g.ks[2]) % g.ks[1], k0 = k / (g.ks[2] * g.ks[1]);
+  const int4 c = in_coords[r];
+  if (c.x != 0 || c.y < 0 || c.y >= g.gi[0] || c.z < 0 || c.z >= g.gi[1] || c.w < 0 || c.w >= g.gi[2]) return;
+  const int t0 = c.y + g.pd[0] - k0 * g.dl[0];
+  const int t1 = c.z + g.pd[1] - k1 * g.dl[1];
+  const int t2 = c.w + g.pd[2] - k2 * g.dl[2];
+  if (t0 < 0 || t1 < 0 || t2 < 0) return;
+  if (t0 % g.st[0] || t1 % g.st[1] || t2 % g.st[2]) return;
+  const int o0 = t0 / g.st[0], o1 = t1 / g.st[1], o2 = t2 / g.st[2];
+  if (o0 >= g.go[0] || o1 >= g.go[1] || o2 >= g.go[2]) return;
+  const uint32_t key = ((uint32_t)o0 * (uint32_t)g.go[1] + (uint32_t)o1) * (uint32_t)g.go[2] + (uint32_t)o2;
+  atomicOr(&bitmap[key >> 5], 1u << (key & 31));
+}
+
+bool Rulebook::init(uint32_t max_in_, uint32_t max_out_, int kvol) {
+  max_in = max_in_;
+  max_out = max_out_;
+  kvol_cap = kvol;
+  ld = (std::max(max_in, max_out) + 63u) & ~63u;
+  if (ld == 0) ld = 64;
+  if (!nbr.alloc((size_t)kvol * ld * sizeof(int32_t))) return false;
+  if (!counters.alloc(64 * sizeof(uint32_t))) return false;
+  if (hipMemset(counters.p, 0, 64 * sizeof(uint32_t)) != hipSuccess) return false;
+  return true;
+}
+
+static int check_geom(const int ks[3], const int st[3], const int dl[3], int kvol_cap) {
+  for (int a = 0; a < 3; ++a)
+    SCN_REQUIRE(ks[a] >= 1 && st[a] >= 1 && dl[a] >= 1, SCN_ERR_INVALID, "kernel/stride/dilation must be >= 1");
+  SCN_REQUIRE(ks[0] * ks[1] * ks[2] <= kvol_cap, SCN_ERR_CAPACITY, "kernel volume %d exceeds the rulebook's %d",
+              ks[0] * ks[1] * ks[2], kvol_cap);
+  return SCN_OK;
+}
+
+
+__global__ void k_set_count(uint32_t* dst, const uint32_t* n_dev, uint32_t n_bound) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    const uint32_t n = eff_n(n_dev, n_bound);
+    dst[0] = n;
+    dst[1] = n;
+  }
+}
+
+static int launch_build_nbr(const Rulebook& rb, const int32_t* out_coords, uint32_t n_bound, bool identity_center,
+                            hipStream_t stream) {
+  if (n_bound == 0) return SCN_OK;
+  hipLaunchKernelGGL(k_build_nbr, dim3(ceil_div(n_bound, 256), rb.geom.kvol), dim3(256), 0, stream,
+                     (const int4*)out_coords, rb.n_out_dev(), n_bound, to_dev(rb.geom), rb.in_table->slots(),
+                     rb.in_table->mask, rb.nbr.as<int32_t>(), rb.ld, identity_center ? 1 : 0);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
+int Rulebook::build_subm(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3], const int ks[3],
+                         const int dil[3], const CoordTable* shared_in_table, hipStream_t stream) {
+  const int one[3] = {1, 1, 1};
+  int rc = check_geom(ks, one, dil, kvol_cap);
+  if (rc) return rc;
+  SCN_REQUIRE(n <= max_in && n <= ld, SCN_ERR_CAPACITY, "submanifold rulebook: %u rows exceed capacity %u", n, max_in);
+  SCN_REQUIRE(grid_fits_u32(grid), SCN_ERR_UNSUPPORTED, "grid %dx%dx%d does not fit 32-bit keys", grid[0], grid[1],
+              grid[2]);
+  subm = true;
+  for (int a = 0; a < 3; ++a) {
+    geom.grid_in[a] = geom.grid_out[a] = grid[a];
+    geom.ks[a] = ks[a];
+    geom.stride[a] = 1;
+    geom.dil[a] = dil[a];
+    geom.pad[a] = (ks[a] / 2) * dil[a];
+  }
+  geom.kvol = ks[0] * ks[1] * ks[2];
+  in_indices = out_indices = idx;
+  n_bound_in = n_bound_out = n;
+  uint32_t* cnt = counters.as<uint32_t>();
+  if (shared_in_table) {
+    in_table = shared_in_table;
+    hipLaunchKernelGGL(k_set_count, dim3(1), dim3(64), 0, stream, cnt, n_dev, n);
+    SCN_HIP(hipGetLastError());
+  } else {
+    if (own_in_table.cap < hash_capacity_for(max_in) && !own_in_table.alloc_for(max_in)) return SCN_ERR_HIP;
+    rc = hash_build(own_in_table, idx, n, n_dev, grid, cnt, stream);
+    if (rc) return rc;
+    in_table = &own_in_table;
+  }
+  const bool odd = (ks[0] & 1) && (ks[1] & 1) && (ks[2] & 1);
+  rc = launch_build_nbr(*this, idx, n, odd, stream);
+  if (rc) return rc;
+  built = true;
+  return SCN_OK;
+}
+
+int Rulebook::build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3], const int ks[3],
+                           const int stride[3], const int pad[3], const int dil[3],
+                           const CoordTable* shared_in_table, hipStream_t stream) {
+  int rc = check_geom(ks, stride, dil, kvol_cap);
+  if (rc) return rc;
+  SCN_REQUIRE(n <= max_in, SCN_ERR_CAPACITY, "sparse rulebook: %u rows exceed capacity %u", n, max_in);
+  SCN_REQUIRE(grid_fits_u32(grid), SCN_ERR_UNSUPPORTED, "grid %dx%dx%d does not fit 32-bit keys", grid[0], grid[1],
+              grid[2]);
+  subm = false;
+  for (int a = 0; a < 3; ++a) {
+    SCN_REQUIRE(pad[a] >= 0, SCN_ERR_INVALID, "negative padding");
+    geom.grid_in[a] = grid[a];
+    geom.ks[a] = ks[a];
+    geom.stride[a] = stride[a];
+    geom.dil[a] = dil[a];
+    geom.pad[a] = pad[a];
+    geom.grid_out[a] = (grid[a] + 2 * pad[a] - dil[a] * (ks[a] - 1) - 1) / stride[a] + 1;
+    SCN_REQUIRE(geom.grid_out[a] >= 1, SCN_ERR_INVALID, "convolution output size < 1 on axis %d", a);
+  }
+  SCN_REQUIRE(grid_fits_u32(geom.grid_out), SCN_ERR_UNSUPPORTED, "output grid does not fit 32-bit keys");
+  geom.kvol = ks[0] * ks[1] * ks[2];
+  in_indices = idx;
+  n_bound_in = n;
+  // host-side bound of the number of outputs
+  {
+    const uint64_t vol = (uint64_t)geom.grid_out[0] * geom.grid_out[1] * geom.grid_out[2];
+    uint64_t b = std::min<uint64_t>((uint64_t)n * (uint64_t)geom.kvol, vol);
+    n_bound_out = (uint32_t)std::min<uint64_t>(b, max_out);
+  }
+  const size_t words = bitmap_words_for(geom.grid_out);
+  if (words != bitmap_words) {
+    if (!bitmap.alloc(words * 4)) return SCN_ERR_HIP;
+    if (!blocksum.alloc((words / kWordsPerBlock + 1) * 4)) return SCN_ERR_HIP;
+    bitmap_words = words;
+  }
+  if (out_idx.bytes < (size_t)max_out * 16 && !out_idx.alloc((size_t)std::max(max_out, 1u) * 16)) return SCN_ERR_HIP;
+  if (out_table.cap < hash_capacity_for(max_out) && !out_table.alloc_for(max_out)) return SCN_ERR_HIP;
+  out_indices = out_idx.as<int32_t>();
+  uint32_t* cnt = counters.as<uint32_t>();
+  // input table
+  if (shared_in_table) {
+    in_table = shared_in_table;
+  } else {
+    if (own_in_table.cap < hash_capacity_for(max_in) && !own_in_table.alloc_for(max_in)) return SCN_ERR_HIP;
+    rc = hash_build(own_in_table, idx, n, n_dev, grid, nullptr, stream);
+    if (rc) return rc;
+    in_table = &own_in_table;
+  }
+  // occupancy bitmap of the outputs -> ordered unique output coordinates + their hash
+  rc = fill_u32(bitmap.p, 0u, words, stream);
+  if (rc) return rc;
+  out_table.mask = (uint32_t)(hash_capacity_for(n_bound_out) - 1);
+  rc = fill_u32(out_table.slots(), 0xFFFFFFFFu, ((size_t)out_table.mask + 1) * 2, stream);
+  if (rc) return rc;
+  const GeomDev gd = to_dev(geom);
+  if (n) {
+    hipLaunchKernelGGL(k_mark_outputs, dim3(ceil_div(n, 256), geom.kvol), dim3(256), 0, stream, (const int4*)idx,
+                       n_dev, n, gd, bitmap.as<uint32_t>());
+  }
+  const uint32_t nblocks = (uint32_t)(words / kWordsPerBlock);
+  hipLaunchKernelGGL(k_bitmap_blocksum, dim3(nblocks), dim3(256), 0, stream, bitmap.as<uint32_t>(),
+                     blocksum.as<uint32_t>());
+  hipLaunchKernelGGL(k_scan_blocksums, dim3(1), dim3(1024), 0, stream, blocksum.as<uint32_t>(), nblocks, cnt,
+                     n_bound_out);
+  hipLaunchKernelGGL(k_bitmap_expand, dim3(nblocks), dim3(256), 0, stream, bitmap.as<uint32_t>(),
+                     blocksum.as<uint32_t>(), Int3{{geom.grid_out[0], geom.grid_out[1], geom.grid_out[2]}},
+                     n_bound_out, (int4*)out_idx.p, out_table.slots(), out_table.mask, (uint32_t*)nullptr);
+  SCN_HIP(hipGetLastError());
+  rc = launch_build_nbr(*this, out_indices, n_bound_out, false, stream);
+  if (rc) return rc;
+  built = true;
+  return SCN_OK;
+}
+
+// ---- pair compaction: nbr[k][o] -> (in,out) lists per offset, ordered by (k, out) -------------
+__global__ __launch_bounds__(256) void k_pair_count(const int32_t* __restrict__ nbr, uint32_t ld,
+                                                    const uint32_t* n_out_dev, uint32_t n_bound, uint32_t* counts) {
+  __shared__ uint32_t wsum[4];
+  const uint32_t n = eff_n(n_out_dev, n_bound);
+  const uint32_t o = blockIdx.x * 256 + threadIdx.x;
+  const bool valid = o < n && nbr[(size_t)blockIdx.y * ld + o] >= 0;
+  const uint64_t m = __ballot(valid);
+  if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = (uint32_t)__popcll(m);
+  __syncthreads();
+  if (threadIdx.x == 0) counts[blockIdx.y * gridDim.x + blockIdx.x] = wsum[0] + wsum[1] + wsum[2] + wsum[3];
+}
+
+__global__ __launch_bounds__(256) void k_pair_write(const int32_t* __restrict__ nbr, uint32_t ld,
+                                                    const uint32_t* n_out_dev, uint32_t n_bound,
+                                                    const uint32_t* __restrict__ block_off, const uint32_t* total,
+                                                    int32_t* pair_in, int32_t* pair_out, int64_t* offsets,
+                                                    uint64_t capacity) {
+  __shared__ uint32_t wsum[4];
+  const uint32_t n = eff_n(n_out_dev, n_bound);
+  const uint32_t o = blockIdx.x * 256 + threadIdx.x;
+  int32_t in = -1;
+  if (o < n) in = nbr[(size_t)blockIdx.y * ld + o];
+  const bool valid = in >= 0;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint64_t m = __ballot(valid);  // wavefront ballot
+  const uint32_t below = (uint32_t)__popcll(m & ((1ull << lane) - 1ull));  // prefix inside the wavefront
+  if (lane == 0) wsum[wave] = (uint32_t)__popcll(m);
+  __syncthreads();
+  uint32_t wbase = 0;
+  for (int w = 0; w < wave; ++w) wbase += wsum[w];
+  const uint32_t base = block_off[blockIdx.y * gridDim.x + blockIdx.x];
+  if (valid) {
+    const uint64_t pos = (uint64_t)base + wbase + below;
+    if (pos < capacity) {
+      pair_in[pos] = in;
+      pair_out[pos] = (int32_t)o;
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    offsets[blockIdx.y] = base;
+    if (blockIdx.y == gridDim.y - 1) offsets[gridDim.y] = total[1];
+  }
+}
+
+int Rulebook::pairs(int32_t* pair_in, int32_t* pair_out, int64_t* offsets, uint64_t capacity, hipStream_t stream) {
+  SCN_REQUIRE(built, SCN_ERR_INVALID, "rulebook has not been built");
+  const uint32_t nb = std::max(1u, ceil_div(n_bound_out, 256));
+  const size_t need = ((size_t)nb * geom.kvol + 8) * 4;
+  if (pair_scratch.bytes < need && !pair_scratch.alloc(need)) return SCN_ERR_HIP;
+  uint32_t* counts = pair_scratch.as<uint32_t>();
+  uint32_t* total = counters.as<uint32_t>() + 8;
+  hipLaunchKernelGGL(k_pair_count, dim3(nb, geom.kvol), dim3(256), 0, stream, nbr.as<int32_t>(), ld, n_out_dev(),
+                     n_bound_out, counts);
+  hipLaunchKernelGGL(k_scan_blocksums, dim3(1), dim3(1024), 0, stream, counts, nb * (uint32_t)geom.kvol, total,
+                     0xFFFFFFFFu);
+  hipLaunchKernelGGL(k_pair_write, dim3(nb, geom.kvol), dim3(256), 0, stream, nbr.as<int32_t>(), ld, n_out_dev(),
+                     n_bound_out, counts, total, pair_in, pair_out, offsets, capacity);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
+// --------------------------------------------------------------------------------------------
+// gather-GEMM convolution
+// --------------------------------------------------------------------------------------------
+// Operand mapping of v_mfma_i32_16x16x64_i8 / v_mfma_f32_16x16x32_f16 (D = A x B + C, wave64):
+//   A (16 x K): lane l supplies row  m = l % 16, the 16 bytes of K-block l / 16
+//   B (K x 16): lane l supplies col  n = l % 16, the 16 bytes of K-block l / 16
+//   D (16 x 16): lane l holds col n = l % 16, rows m = 4 * (l / 16) + {0,1,2,3}
+// Rows of A are output channels (weights, pre-packed on the host in exactly this order), columns of
+// B are voxels: the 16 bytes a lane needs are 16 contiguous input channels of one gathered row, so
+// a gathered row goes from memory straight into the MFMA operand with one 16-byte load, and each
+// lane ends up with 4 consecutive output channels of one voxel, stored with one 4/8-byte store.
+// One 16-byte "chunk" = 16 int8 or 8 fp16 input channels; K-step s consumes chunks 4s..4s+3 of the
+// sequence (offset 0 chunk 0, offset 0 chunk 1, ..., offset kvol-1 chunk CHUNKS-1).
+struct ConvArgs {
+  const char* x;
+  uint32_t x_ld_bytes;
+  const int32_t* nbr;
+  uint32_t nbr_ld;
+  int kvol;
+  const uint32_t* n_out_dev;
+  uint32_t n_bound;
+  const uint4* wfrag;
+  int steps;
+  const float* wscale;
+  const float* bias;
+  int cout;
+  float x_scale;
+  int relu;
+  int out_dtype;
+  float out_scale;
+  char* out;
+  uint32_t out_ld;
+  void* acc;
+  const char* res;
+  int res_dtype;
+  float res_scale;
+  uint32_t res_ld;
+  int mid_dtype;
+  float mid_scale;
+  float a_rq, b_rq;
+  int relu2;
+};
+
+__device__ __forceinline__ float quant_f(float y, float s) {
+  float q = rintf(y / s);
+  q = fminf(fmaxf(q, -127.f), 127.f);  // NaN -> -127 (fmaxf returns the non-NaN operand)
+  return q;
+}
+
+__device__ __forceinline__ float half_round(float y) { return (float)(_Float16)y; }
+
+template <int EL>
+struct Mma;
+template <>
+struct Mma<0> {
+  using Acc = v4i;
+  static __device__ __forceinline__ Acc run(const uint4& a, const uint4& b, Acc c) {
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, a), __builtin_bit_cast(v4i, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<1> {
+  using Acc = v4f;
+  static __device__ __forceinline__ Acc run(const uint4& a, const uint4& b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+};
+
+// Stores 4 consecutive channels of one row after the fused epilogue.
+template <int EL>
+__device__ __forceinline__ void epilogue_store(const ConvArgs& a, uint32_t row, int co, const typename Mma<EL>::Acc& acc) {
+  float y[4];
+  const float4 bs = *reinterpret_cast<const float4*>(a.bias + co);
+  const float b4[4] = {bs.x, bs.y, bs.z, bs.w};
+  if (EL == 0) {
+    const float4 ws = *reinterpret_cast<const float4*>(a.wscale + co);
+    const float w4[4] = {ws.x, ws.y, ws.z, ws.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float sc = a.x_scale * w4[j];         // s_x * s_w[c], one fp32 rounding
+      const float m = (float)acc[j] * sc;          // fp32 multiply
+      y[j] = m + b4[j];                            // fp32 add (the library is built with -ffp-contract=off)
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) y[j] = (float)acc[j] + b4[j];
+  }
+  if (a.acc) {
+    if (EL == 0)
+      *reinterpret_cast<v4i*>((int32_t*)a.acc + (size_t)row * a.cout + co) = __builtin_bit_cast(v4i, acc);
+    else
+      *reinterpret_cast<v4f*>((float*)a.acc + (size_t)row * a.cout + co) = __builtin_bit_cast(v4f, acc);
+  }
+  if (a.relu) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) y[j] = y[j] > 0.f ? y[j] : 0.f;
+  }
+  if (a.res) {
+    // value of the un-fused conv output as its consumer (the Add) would have read it
+    float rv[4];
+    if (a.res_dtype == SCN_DTYPE_INT8) {
+      const char4 r = *reinterpret_cast<const char4*>(a.res + (size_t)row * a.res_ld + co);
+      rv[0] = (float)r.x * a.res_scale;
+      rv[1] = (float)r.y * a.res_scale;
+      rv[2] = (float)r.z * a.res_scale;
+      rv[3] = (float)r.w * a.res_scale;
+    } else {
+      const _Float16* r = reinterpret_cast<const _Float16*>(a.res) + (size_t)row * a.res_ld + co;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        rv[j] = (float)r[j];
+        if (a.b_rq > 0.f) rv[j] = quant_f(rv[j], a.b_rq) * a.b_rq;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float v;
+      if (a.mid_dtype == SCN_DTYPE_INT8) {
+        v = quant_f(y[j], a.mid_scale) * a.mid_scale;
+      } else {
+        v = half_round(y[j]);
+        if (a.a_rq > 0.f) v = quant_f(v, a.a_rq) * a.a_rq;
+      }
+      v = v + rv[j];
+      if (a.relu2) v = v > 0.f ? v : 0.f;
+      y[j] = v;
+    }
+  }
+  if (a.out_dtype == SCN_DTYPE_INT8) {
+    char4 q;
+    q.x = (signed char)quant_f(y[0], a.out_scale);
+    q.y = (signed char)quant_f(y[1], a.out_scale);
+    q.z = (signed char)quant_f(y[2], a.out_scale);
+    q.w = (signed char)quant_f(y[3], a.out_scale);
+    *reinterpret_cast<char4*>(a.out + (size_t)row * a.out_ld + co) = q;
+  } else {
+    typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+    v4h h = {(_Float16)y[0], (_Float16)y[1], (_Float16)y[2], (_Float16)y[3]};
+    *reinterpret_cast<v4h*>(reinterpret_cast<_Float16*>(a.out) + (size_t)row * a.out_ld + co) = h;
+  }
+}
+
+// Row-split kernel: each wave owns 16*NT output rows and all MT*16 output channels; both operands
+// come straight from global memory / L2 (weights: coalesced 1 KB fragments; features: gathered rows).
+template <int EL, int CHUNKS, int MT, int NT>
+__global__ __launch_bounds__(256) void k_conv_rows(const ConvArgs a) {
+  using Acc = typename Mma<EL>::Acc;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const uint32_t n = eff_n(a.n_out_dev, a.n_bound);
+  const uint32_t row0 = (blockIdx.x * 4 + wave) * (16 * NT);
+  if (row0 >= n) return;
+  Acc acc[MT][NT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int u = 0; u < NT; ++u) acc[t][u] = Acc{0, 0, 0, 0};
+  const uint4* wf = a.wfrag + lane;
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  uint32_t rows[NT];
+#pragma unroll
+  for (int u = 0; u < NT; ++u) rows[u] = row0 + u * 16 + lr;
+
+  if constexpr (CHUNKS >= 4) {
+    constexpr int SPK = CHUNKS / 4;  // K-steps per kernel offset
+    for (int k = 0; k < a.kvol; ++k) {
+      int32_t idx[NT];
+      bool any = false;
+#pragma unroll
+      for (int u = 0; u < NT; ++u) {
+        idx[u] = rows[u] < n ? a.nbr[(size_t)k * a.nbr_ld + rows[u]] : -1;
+        any |= idx[u] >= 0;
+      }
+      if (!__any(any)) continue;  // no row of this wave has a neighbour at this offset
+#pragma unroll
+      for (int ss = 0; ss < SPK; ++ss) {
+        uint4 b[NT];
+#pragma unroll
+        for (int u = 0; u < NT; ++u)
+          b[u] = idx[u] >= 0
+                     ? *reinterpret_cast<const uint4*>(a.x + (size_t)idx[u] * a.x_ld_bytes + (ss * 4 + lg) * 16)
+                     : zero;
+        const int s = k * SPK + ss;
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          const uint4 av = wf[(size_t)(s * MT + t) * 64];
+#pragma unroll
+          for (int u = 0; u < NT; ++u) acc[t][u] = Mma<EL>::run(av, b[u], acc[t][u]);
+        }
+      }
+    }
+  } else {
+    const int total_chunks = a.kvol * CHUNKS;
+    for (int s = 0; s < a.steps; ++s) {
+      const int g = 4 * s + lg;
+      const int k = g / CHUNKS, c = g % CHUNKS;
+      const bool gv = g < total_chunks;
+      uint4 b[NT];
+      bool any = false;
+#pragma unroll
+      for (int u = 0; u < NT; ++u) {
+        int32_t idx = -1;
+        if (gv && rows[u] < n) idx = a.nbr[(size_t)k * a.nbr_ld + rows[u]];
+        any |= idx >= 0;
+        b[u] = idx >= 0 ? *reinterpret_cast<const uint4*>(a.x + (size_t)idx * a.x_ld_bytes + c * 16) : zero;
+      }
+      if (!__any(any)) continue;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const uint4 av = wf[(size_t)(s * MT + t) * 64];
+#pragma unroll
+        for (int u = 0; u < NT; ++u) acc[t][u] = Mma<EL>::run(av, b[u], acc[t][u]);
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < NT; ++u) {
+    if (rows[u] >= n) continue;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) epilogue_store<EL>(a, rows[u], t * 16 + lg * 4, acc[t][u]);
+  }
+}
+
+bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* ranges, const uint16_t* bias_fp16,
+                       int prec) {
+  cout = shape[0];
+  ks[0] = shape[1];
+  ks[1] = shape[2];
+  ks[2] = shape[3];
+  cin = shape[4];
+  kvol = ks[0] * ks[1] * ks[2];
+  precision = prec;
+  if (cout <= 0 || cin <= 0 || kvol <= 0) {
+    set_error("invalid weight shape");
+    return false;
+  }
+  if (prec == SCN_PRECISION_INT8 && ranges == nullptr) {
+    set_error("int8 convolution needs weight_dynamic_ranges");
+    return false;
+  }
+  const int epc = prec == SCN_PRECISION_INT8 ? 16 : 8;  // elements per 16-byte chunk
+  int ch = (cin + epc - 1) / epc;
+  int p2 = 1;
+  while (p2 < ch) p2 <<= 1;  // chunks per row rounded to a power of two (rows are padded to it)
+  chunks = p2;
+  cin_pad = (uint32_t)(chunks * epc);
+  mtiles = (cout + 15) / 16;
+  steps = (kvol * chunks + 3) / 4;
+  const int cout_pad = mtiles * 16;
+  std::vector<float> ws(cout_pad, 1.f), bs(cout_pad, 0.f);
+  for (int c = 0; c < cout; ++c) {
+    if (prec == SCN_PRECISION_INT8) ws[c] = ranges[c] / 127.f;
+    if (bias_fp16) bs[c] = half_bits_to_float(bias_fp16[c]);
+  }
+  std::vector<uint8_t> frag((size_t)steps * mtiles * 64 * 16, 0);
+  for (int s = 0; s < steps; ++s)
+    for (int t = 0; t < mtiles; ++t)
+      for (int l = 0; l < 64; ++l) {
+        const int g = 4 * s + l / 16;
+        if (g >= kvol * chunks) continue;
+        const int k = g / chunks, c = g % chunks;
+        const int co = 16 * t + l % 16;
+        if (co >= cout) continue;
+        uint8_t* dst = &frag[((size_t)(s * mtiles + t) * 64 + l) * 16];
+        for (int e = 0; e < epc; ++e) {
+          const int ci = c * epc + e;
+          if (ci >= cin) break;
+          const uint16_t hb = w_fp16[((size_t)co * kvol + k) * cin + ci];
+          if (prec == SCN_PRECISION_INT8) {
+            float q = rintf(half_bits_to_float(hb) / ws[co]);
+            if (!(q >= -127.f)) q = -127.f;
+            if (q > 127.f) q = 127.f;
+            dst[e] = (uint8_t)(int8_t)q;
+          } else {
+            memcpy(dst + 2 * e, &hb, 2);
+          }
+        }
+      }
+  if (!wfrag.alloc(frag.size()) || !wscale.alloc(ws.size() * 4) || !bias.alloc(bs.size() * 4)) return false;
+  if (hipMemcpy(wfrag.p, frag.data(), frag.size(), hipMemcpyHostToDevice) != hipSuccess ||
+      hipMemcpy(wscale.p, ws.data(), ws.size() * 4, hipMemcpyHostToDevice) != hipSuccess ||
+      hipMemcpy(bias.p, bs.data(), bs.size() * 4, hipMemcpyHostToDevice) != hipSuccess) {
+    set_error("weight upload failed");
+    return false;
+  }
+  return true;
+}
+
+template <int EL, int CHUNKS, int MT>
+static void launch_conv_rows(const ConvArgs& a, hipStream_t stream) {
+  constexpr int NT = MT >= 8 ? 2 : 4;
+  const uint32_t rows_per_block = 4 * 16 * NT;
+  hipLaunchKernelGGL((k_conv_rows<EL, CHUNKS, MT, NT>), dim3(ceil_div(a.n_bound, rows_per_block)), dim3(256), 0, stream,
+                     a);
+}
+
+template <int EL, int CHUNKS>
+static bool dispatch_mt(int mt, const ConvArgs& a, hipStream_t stream) {
+  switch (mt) {
+    case 1: launch_conv_rows<EL, CHUNKS, 1>(a, stream); return true;
+    case 2: launch_conv_rows<EL, CHUNKS, 2>(a, stream); return true;
+    case 4: launch_conv_rows<EL, CHUNKS, 4>(a, stream); return true;
+    case 8: launch_conv_rows<EL, CHUNKS, 8>(a, stream); return true;
+    default: return false;
+  }
+}
+
+template <int EL>
+static bool dispatch_chunks(int chunks, int mt, const ConvArgs& a, hipStream_t stream) {
+  switch (chunks) {
+    case 1: return dispatch_mt<EL, 1>(mt, a, stream);
+    case 2: return dispatch_mt<EL, 2>(mt, a, stream);
+    case 4: return dispatch_mt<EL, 4>(mt, a, stream);
+    case 8: return dispatch_mt<EL, 8>(mt, a, stream);
+    case 16: return dispatch_mt<EL, 16>(mt, a, stream);
+    default: return false;
+  }
+}
+
+int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, const uint32_t* n_out_dev,
+                 uint32_t n_bound, const scn_conv_io& io, hipStream_t stream) {
+  if (n_bound == 0) return SCN_OK;
+  const int esz = w.precision == SCN_PRECISION_INT8 ? 1 : 2;
+  SCN_REQUIRE(io.x_dev && io.out_dev, SCN_ERR_INVALID, "conv: null input or output");
+  SCN_REQUIRE(io.x_ld >= w.cin_pad, SCN_ERR_INVALID, "conv: input row stride %u < padded channels %u", io.x_ld,
+              w.cin_pad);
+  SCN_REQUIRE(((size_t)io.x_ld * esz) % 16 == 0 && ((uintptr_t)io.x_dev & 15) == 0, SCN_ERR_INVALID,
+              "conv: input rows must be 16-byte aligned");
+  SCN_REQUIRE(io.out_dtype == SCN_DTYPE_INT8 || io.out_dtype == SCN_DTYPE_FP16, SCN_ERR_INVALID, "conv: bad out dtype");
+  SCN_REQUIRE(io.out_ld >= (uint32_t)w.mtiles * 16, SCN_ERR_INVALID, "conv: output row stride %u < %d", io.out_ld,
+              w.mtiles * 16);
+  const int osz = io.out_dtype == SCN_DTYPE_INT8 ? 1 : 2;
+  SCN_REQUIRE(((size_t)io.out_ld * osz) % (4 * osz) == 0 && ((uintptr_t)io.out_dev & 7) == 0, SCN_ERR_INVALID,
+              "conv: output rows must be 8-byte aligned");
+  if (io.res_dev) {
+    SCN_REQUIRE(io.res_dtype == SCN_DTYPE_INT8 || io.res_dtype == SCN_DTYPE_FP16, SCN_ERR_INVALID, "conv: bad residual dtype");
+    SCN_REQUIRE(io.mid_dtype == SCN_DTYPE_INT8 || io.mid_dtype == SCN_DTYPE_FP16, SCN_ERR_INVALID, "conv: bad mid dtype");
+    SCN_REQUIRE(io.res_ld >= (uint32_t)w.mtiles * 16 && io.res_ld % 4 == 0 && ((uintptr_t)io.res_dev & 7) == 0,
+                SCN_ERR_INVALID, "conv: residual rows misaligned or too short");
+  }
+  SCN_REQUIRE(!io.acc_dev || w.cout % 16 == 0, SCN_ERR_UNSUPPORTED, "accumulator dump needs Cout %% 16 == 0");
+  ConvArgs a;
+  a.x = (const char*)io.x_dev;
+  a.x_ld_bytes = io.x_ld * esz;
+  a.nbr = nbr;
+  a.nbr_ld = nbr_ld;
+  a.kvol = w.kvol;
+  a.n_out_dev = n_out_dev;
+  a.n_bound = n_bound;
+  a.wfrag = w.wfrag.as<uint4>();
+  a.steps = w.steps;
+  a.wscale = w.wscale.as<float>();
+  a.bias = w.bias.as<float>();
+  a.cout = w.cout;
+  a.x_scale = io.x_scale;
+  a.relu = io.relu;
+  a.out_dtype = io.out_dtype;
+  a.out_scale = io.out_scale;
+  a.out = (char*)io.out_dev;
+  a.out_ld = io.out_ld;
+  a.acc = io.acc_dev;
+  a.res = (const char*)io.res_dev;
+  a.res_dtype = io.res_dtype;
+  a.res_scale = io.res_scale;
+  a.res_ld = io.res_ld;
+  a.mid_dtype = io.mid_dtype;
+  a.mid_scale = io.mid_scale;
+  a.a_rq = io.a_requant_scale;
+  a.b_rq = io.b_requant_scale;
+  a.relu2 = io.relu_after_add;
+  bool ok = w.precision == SCN_PRECISION_INT8 ? dispatch_chunks<0>(w.chunks, w.mtiles, a, stream)
+                                               : dispatch_chunks<1>(w.chunks, w.mtiles, a, stream);
+  SCN_REQUIRE(ok, SCN_ERR_UNSUPPORTED, "conv: no kernel for Cin=%d Cout=%d (chunks %d, m-tiles %d)", w.cin, w.cout,
+              w.chunks, w.mtiles);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
+// --------------------------------------------------------------------------------------------
+// elementwise glue
+// --------------------------------------------------------------------------------------------
+__device__ __forceinline__ float load_value(const void* p, int dtype, size_t i, float scale, float rq) {
+  if (dtype == SCN_DTYPE_INT8) return (float)reinterpret_cast<const signed char*>(p)[i] * scale;
+  float v = (float)reinterpret_cast<const _Float16*>(p)[i];
+  if (rq > 0.f) v = quant_f(v, rq) * rq;
+  return v;
+}
+
+__device__ __forceinline__ void store_value(void* p, int dtype, size_t i, float v, float scale) {
+  if (dtype == SCN_DTYPE_INT8)
+    reinterpret_cast<signed char*>(p)[i] = (signed char)quant_f(v, scale);
+  else
+    reinterpret_cast<_Float16*>(p)[i] = (_Float16)v;
+}
+
+__global__ __launch_bounds__(256) void k_convert_rows(const void* in, int in_dtype, uint32_t in_c, uint32_t in_ld,
+                                                      float in_scale, void* out, int out_dtype, uint32_t out_c,
+                                                      uint32_t out_ld, float out_scale, int relu, uint32_t n_bound,
+                                                      const uint32_t* n_dev) {
+  const uint32_t n = eff_n(n_dev, n_bound);
+  const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const uint32_t row = (uint32_t)(t / out_c), c = (uint32_t)(t % out_c);
+  if (row >= n) return;
+  float v = 0.f;
+  if (c < in_c) v = load_value(in, in_dtype, (size_t)row * in_ld + c, in_scale, 0.f);
+  if (relu) v = v > 0.f ? v : 0.f;
+  store_value(out, out_dtype, (size_t)row * out_ld + c, v, out_scale);
+}
+
+int convert_rows(const void* in, int in_dtype, uint32_t in_c, uint32_t in_ld, float in_scale, void* out,
+                 int out_dtype, uint32_t out_c, uint32_t out_ld, float out_scale, int relu, uint32_t n,
+                 const uint32_t* n_dev, hipStream_t stream) {
+  if (n == 0) return SCN_OK;
+  SCN_REQUIRE(in && out && out_c > 0 && out_ld >= out_c && in_ld >= in_c, SCN_ERR_INVALID, "convert_rows: bad arguments");
+  const size_t total = (size_t)n * out_c;
+  hipLaunchKernelGGL(k_convert_rows, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, in, in_dtype, in_c,
+                     in_ld, in_scale, out, out_dtype, out_c, out_ld, out_scale, relu, n, n_dev);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
+__global__ __launch_bounds__(256) void k_add_relu(const void* a, int a_dtype, float a_scale, float a_rq, const void* b,
+                                                  int b_dtype, float b_scale, float b_rq, void* out, int out_dtype,
+                                                  float out_scale, int relu, uint32_t c, uint32_t n_bound,
+                                                  const uint32_t* n_dev) {
+  const size_t total = (size_t)eff_n(n_dev, n_bound) * c;
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  float v = load_value(a, a_dtype, i, a_scale, a_rq) + load_value(b, b_dtype, i, b_scale, b_rq);
+  if (relu) v = v > 0.f ? v : 0.f;
+  store_value(out, out_dtype, i, v, out_scale);
+}
+
+int add_relu(const void* a, int a_dtype, float a_scale, float a_rq, const void* b, int b_dtype, float b_scale,
+             float b_rq, void* out, int out_dtype, float out_scale, int relu, uint32_t c, uint32_t n,
+             const uint32_t* n_dev, hipStream_t stream) {
+  if (n == 0 || c == 0) return SCN_OK;
+  SCN_REQUIRE(a && b && out, SCN_ERR_INVALID, "add_relu: null pointer");
+  const size_t total = (size_t)n * c;
+  hipLaunchKernelGGL(k_add_relu, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, a_dtype, a_scale, a_rq,
+                     b, b_dtype, b_scale, b_rq, out, out_dtype, out_scale, relu, c, n, n_dev);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
+// --------------------------------------------------------------------------------------------
+// sparse -> dense.  strides are those of the final (possibly transposed) layout, in elements.
+// --------------------------------------------------------------------------------------------
+struct DenseStrides {
+  int64_t sc, s0, s1, s2;
+  int d0, d1, d2;
+};
+
+__global__ __launch_bounds__(256) void k_scatter_dense(const void* feat, int dtype, float scale, uint32_t ld,
+                                                       const int4* __restrict__ coords, uint32_t n_bound,
+                                                       const uint32_t* n_dev, DenseStrides st, _Float16* out) {
+  const uint32_t n = eff_n(n_dev, n_bound);
+  const uint32_t row = blockIdx.x * 256 + threadIdx.x;
+  if (row >= n) return;
+  const uint32_t c = blockIdx.y;
+  const int4 p = coords[row];
+  if (p.x != 0 || p.y < 0 || p.y >= st.d0 || p.z < 0 || p.z >= st.d1 || p.w < 0 || p.w >= st.d2) return;
+  const float v = load_value(feat, dtype, (size_t)row * ld + c, scale, 0.f);
+  out[c * st.sc + p.y * st.s0 + p.z * st.s1 + p.w * st.s2] = (_Float16)v;
+}
+
+int scatter_dense(const void* feat, int dtype, float scale, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
+                  const uint32_t* n_dev, const int dense_shape[5], const int perm[5], void* out, hipStream_t stream) {
+  SCN_REQUIRE(out && dense_shape, SCN_ERR_INVALID, "scatter_dense: null pointer");
+  SCN_REQUIRE(dense_shape[0] == 1 && (uint32_t)dense_shape[1] == c, SCN_ERR_INVALID,
+              "scatter_dense: output_shape must be [1, C=%u, D0, D1, D2]", c);
+  int p[5] = {0, 1, 2, 3, 4};
+  if (perm) {
+    bool seen[5] = {false, false, false, false, false};
+    for (int j = 0; j < 5; ++j) {
+      SCN_REQUIRE(perm[j] >= 0 && perm[j] < 5 && !seen[perm[j]], SCN_ERR_INVALID, "scatter_dense: bad permutation");
+      seen[perm[j]] = true;
+      p[j] = perm[j];
+    }
+  }
+  int64_t tstride[5];
+  int64_t s = 1;
+  for (int j = 4; j >= 0; --j) {
+    tstride[j] = s;
+    s *= dense_shape[p[j]];
+  }
+  int64_t dstride[5];
+  for (int j = 0; j < 5; ++j) dstride[p[j]] = tstride[j];
+  const size_t numel = (size_t)s;
+  SCN_REQUIRE(numel % 2 == 0, SCN_ERR_UNSUPPORTED, "scatter_dense: odd element count");
+  int rc = fill_u32(out, 0u, numel / 2, stream);
+  if (rc) return rc;
+  if (n == 0) return SCN_OK;
+  SCN_REQUIRE(feat && idx, SCN_ERR_INVALID, "scatter_dense: null input");
+  DenseStrides st{dstride[1], dstride[2], dstride[3], dstride[4], dense_shape[2], dense_shape[3], dense_shape[4]};
+  hipLaunchKernelGGL(k_scatter_dense, dim3(ceil_div(n, 256), c), dim3(256), 0, stream, feat, dtype, scale, ld,
+                     (const int4*)idx, n, n_dev, st, (_Float16*)out);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
+// --------------------------------------------------------------------------------------------
+// voxelization
+// --------------------------------------------------------------------------------------------
+struct VoxGeom {
+  float mn[3], mx[3], vs[3];
+  int g[3];     // x, y, z cells
+  int og[3];    // grid in output coordinate order (zyx: z,y,x / xyz: x,y,z)
+  int order;
+  int nf;
+  int max_voxels, max_pts;
+};
+
+// Pass 1 over the point stream: cell key per point + occupancy bit.
+__global__ __launch_bounds__(256) void k_vox_mark(const _Float16* __restrict__ pts, uint32_t n, VoxGeom g,
+                                                  uint32_t* pkey, uint32_t* bitmap) {
+  const uint32_t p = blockIdx.x * 256 + threadIdx.x;
+  if (p >= n) return;
+  const float px = (float)pts[(size_t)p * g.nf + 0];
+  const float py = (float)pts[(size_t)p * g.nf + 1];
+  const float pz = (float)pts[(size_t)p * g.nf + 2];
+  uint32_t key = 0xFFFFFFFFu;
+  if (px >= g.mn[0] && px < g.mx[0] && py >= g.mn[1] && py < g.mx[1] && pz >= g.mn[2] && pz < g.mx[2]) {
+    const int ix = (int)floorf((px - g.mn[0]) / g.vs[0]);
+    const int iy = (int)floorf((py - g.mn[1]) / g.vs[1]);
+    const int iz = (int)floorf((pz - g.mn[2]) / g.vs[2]);
+    if (ix >= 0 && ix < g.g[0] && iy >= 0 && iy < g.g[1] && iz >= 0 && iz < g.g[2]) {
+      key = g.order == SCN_ORDER_ZYX ? ((uint32_t)iz * g.g[1] + iy) * g.g[0] + ix
+                                     : ((uint32_t)ix * g.g[1] + iy) * g.g[2] + iz;
+      atomicOr(&bitmap[key >> 5], 1u << (key & 31));
+    }
+  }
+  pkey[p] = key;
+}
+
+// Pass 2: voxel id = rank of the cell; count the point and keep the max_pts lowest point indices
+// of the voxel, sorted, with an atomicMin cascade (slot j ends up holding the j-th smallest index
+// whatever the arrival order).
+__global__ __launch_bounds__(256) void k_vox_assign(const uint32_t* __restrict__ pkey, uint32_t n,
+                                                    const uint32_t* __restrict__ bitmap,
+                                                    const uint32_t* __restrict__ prefix, int max_voxels, int max_pts,
+                                                    uint32_t* counts, uint32_t* mins) {
+  const uint32_t p = blockIdx.x * 256 + threadIdx.x;
+  if (p >= n) return;
+  const uint32_t key = pkey[p];
+  if (key == 0xFFFFFFFFu) return;
+  const uint32_t w = key >> 5, b = key & 31;
+  const uint32_t id = prefix[w] + __popc(bitmap[w] & ((1u << b) - 1u));
+  if (id >= (uint32_t)max_voxels) return;
+  atomicAdd(&counts[id], 1u);
+  uint32_t x = p;
+  uint32_t* slot = mins + (size_t)id * max_pts;
+  for (int j = 0; j < max_pts; ++j) {
+    const uint32_t old = atomicMin(&slot[j], x);
+    if (old == 0xFFFFFFFFu) break;  // slot was empty: nothing is displaced
+    x = old > x ? old : x;
+  }
+}
+
+// Pass 3: per voxel mean of the kept points, summed in point-index order in fp32.
+__global__ __launch_bounds__(256) void k_vox_mean(const _Float16* __restrict__ pts, const uint32_t* n_vox_dev,
+                                                  int max_voxels, int max_pts, int nf,
+                                                  const uint32_t* __restrict__ counts,
+                                                  const uint32_t* __restrict__ mins, _Float16* feats) {
+  const uint32_t nv = eff_n(n_vox_dev, (uint32_t)max_voxels);
+  const uint32_t t = blockIdx.x * 256 + threadIdx.x;
+  const uint32_t v = t / nf, f = t % nf;
+  if (v >= nv) return;
+  uint32_t cnt = counts[v];
+  if (cnt > (uint32_t)max_pts) cnt = max_pts;
+  const uint32_t* slot = mins + (size_t)v * max_pts;
+  float s = 0.f;
+  for (uint32_t j = 0; j < cnt; ++j) {
+    const float x = (float)pts[(size_t)slot[j] * nf + f];
+    s = j == 0 ? x : s + x;
+  }
+  s = s / (float)cnt;
+  feats[(size_t)v * nf + f] = (_Float16)s;
+}
+
+}  // namespace scn
+
+// ============================================================================================
+// C ABI: stage-level entry points
+// ============================================================================================
+using namespace scn;
+
+extern "C" {
+
+uint64_t scn_hash_u64(uint64_t key) { return hash64(key); }
+size_t scn_hash_capacity_for(uint32_t n) { return hash_capacity_for(n); }
+
+int scn_hash_build(uint64_t* table_dev, size_t capacity, const int32_t* indices_dev, uint32_t n,
+                   const uint32_t* n_dev, const int grid[3], void* stream) {
+  SCN_REQUIRE(table_dev && grid && (indices_dev || n == 0), SCN_ERR_INVALID, "scn_hash_build: null pointer");
+  SCN_REQUIRE(capacity >= hash_capacity_for(n) && (capacity & (capacity - 1)) == 0, SCN_ERR_CAPACITY,
+              "scn_hash_build: capacity %zu must be a power of two >= %zu", capacity, hash_capacity_for(n));
+  SCN_REQUIRE(grid_fits_u32(grid), SCN_ERR_UNSUPPORTED, "grid does not fit 32-bit keys");
+  // the whole caller-provided table is used so that scn_hash_query can be given the same capacity
+  int rc = fill_u32(table_dev, 0xFFFFFFFFu, capacity * 2, (hipStream_t)stream);
+  if (rc) return rc;
+  Int3 g{{grid[0], grid[1], grid[2]}};
+  if (n) {
+    hipLaunchKernelGGL(k_hash_insert, dim3(ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, table_dev,
+                       (uint32_t)(capacity - 1), (const int4*)indices_dev, n, n_dev, g, (uint32_t*)nullptr);
+    SCN_HIP(hipGetLastError());
+  }
+  return SCN_OK;
+}
+
+int scn_hash_query(const uint64_t* table_dev, size_t capacity, const int32_t* coords_dev, uint32_t n,
+                   const int grid[3], int32_t* rows_out_dev, void* stream) {
+  SCN_REQUIRE(table_dev && grid && rows_out_dev && (coords_dev || n == 0), SCN_ERR_INVALID, "scn_hash_query: null pointer");
+  SCN_REQUIRE(capacity && (capacity & (capacity - 1)) == 0, SCN_ERR_INVALID, "capacity must be a power of two");
+  if (n == 0) return SCN_OK;
+  Int3 g{{grid[0], grid[1], grid[2]}};
+  hipLaunchKernelGGL(k_hash_query, dim3(ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, table_dev,
+                     (uint32_t)(capacity - 1), (const int4*)coords_dev, n, g, rows_out_dev);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
+// ---- voxelizer ------------------------------------------------------------------------------
+scn_voxelizer* scn_voxelizer_create(const scn_voxelization_param* param) {
+  if (!param || param->num_feature < 3 || param->max_voxels <= 0 || param->max_points_per_voxel <= 0 ||
+      param->max_points <= 0) {
+    set_error("scn_voxelizer_create: invalid parameter");
+    return nullptr;
+  }
+  const int g[3] = {param->grid_size[0], param->grid_size[1], param->grid_size[2]};
+  if (!grid_fits_u32(g)) {
+    set_error("scn_voxelizer_create: grid does not fit 32-bit keys");
+    return nullptr;
+  }
+  auto* v = new scn_voxelizer();
+  v->p = *param;
+  v->words = bitmap_words_for(g);
+  const size_t mv = (size_t)param->max_voxels;
+  bool ok = v->bitmap.alloc(v->words * 4) && v->prefix.alloc(v->words * 4) &&
+            v->blocksum.alloc((v->words / kWordsPerBlock + 1) * 4) && v->pkey.alloc((size_t)param->max_points * 4) &&
+            v->mins.alloc(mv * param->max_points_per_voxel * 4) && v->counts.alloc(mv * 4) &&
+            v->feats.alloc(mv * param->num_feature * 2) && v->idx.alloc(mv * 16) && v->counters.alloc(64);
+  if (ok) ok = hipMemset(v->counters.p, 0, 64) == hipSuccess && hipMemset(v->idx.p, 0, mv * 16) == hipSuccess &&
+               hipMemset(v->feats.p, 0, mv * param->num_feature * 2) == hipSuccess &&
+               hipHostMalloc((void**)&v->host_count, sizeof(uint32_t), hipHostMallocDefault) == hipSuccess;
+  if (!ok) {
+    delete v;
+    return nullptr;
+  }
+  *v->host_count = 0;
+  return v;
+}
+
+void scn_voxelizer_destroy(scn_voxelizer* v) {
+  if (!v) return;
+  if (v->host_count) (void)hipHostFree(v->host_count);
+  delete v;
+}
+
+int scn_voxelizer_forward(scn_voxelizer* v, const void* points_fp16_dev, uint32_t num_points, int order,
+                          void* stream_) {
+  SCN_REQUIRE(v, SCN_ERR_INVALID, "scn_voxelizer_forward: null voxelizer");
+  SCN_REQUIRE(order == SCN_ORDER_XYZ || order == SCN_ORDER_ZYX, SCN_ERR_INVALID, "Invalid output_order: %d", order);
+  SCN_REQUIRE(points_fp16_dev || num_points == 0, SCN_ERR_INVALID, "scn_voxelizer_forward: null points");
+  hipStream_t stream = (hipStream_t)stream_;
+  if (num_points > (uint32_t)v->p.max_points) {
+    SCN_LOGW("voxelization: %u points exceed max_points %d, the frame is cropped", num_points, v->p.max_points);
+    num_points = (uint32_t)v->p.max_points;
+  }
+  const auto& p = v->p;
+  VoxGeom g;
+  for (int a = 0; a < 3; ++a) {
+    g.mn[a] = p.min_range[a];
+    g.mx[a] = p.max_range[a];
+    g.vs[a] = p.voxel_size[a];
+    g.g[a] = p.grid_size[a];
+  }
+  g.order = order;
+  if (order == SCN_ORDER_ZYX) {
+    g.og[0] = p.grid_size[2]; g.og[1] = p.grid_size[1]; g.og[2] = p.grid_size[0];
+  } else {
+    g.og[0] = p.grid_size[0]; g.og[1] = p.grid_size[1]; g.og[2] = p.grid_size[2];
+  }
+  g.nf = p.num_feature;
+  g.max_voxels = p.max_voxels;
+  g.max_pts = p.max_points_per_voxel;
+  v->last_order = order;
+  int rc = fill_u32(v->bitmap.p, 0u, v->words, stream);
+  if (rc) return rc;
+  rc = fill_u32(v->mins.p, 0xFFFFFFFFu, (size_t)p.max_voxels * p.max_points_per_voxel, stream);
+  if (rc) return rc;
+  rc = fill_u32(v->counts.p, 0u, (size_t)p.max_voxels, stream);
+  if (rc) return rc;
+  uint32_t* cnt = v->counters.as<uint32_t>();
+  const uint32_t nblocks = (uint32_t)(v->words / kWordsPerBlock);
+  if (num_points)
+    hipLaunchKernelGGL(k_vox_mark, dim3(ceil_div(num_points, 256)), dim3(256), 0, stream,
+                       (const _Float16*)points_fp16_dev, num_points, g, v->pkey.as<uint32_t>(), v->bitmap.as<uint32_t>());
+  hipLaunchKernelGGL(k_bitmap_blocksum, dim3(nblocks), dim3(256), 0, stream, v->bitmap.as<uint32_t>(),
+                     v->blocksum.as<uint32_t>());
+  hipLaunchKernelGGL(k_scan_blocksums, dim3(1), dim3(1024), 0, stream, v->blocksum.as<uint32_t>(), nblocks, cnt,
+                     (uint32_t)p.max_voxels);
+  hipLaunchKernelGGL(k_bitmap_expand, dim3(nblocks), dim3(256), 0, stream, v->bitmap.as<uint32_t>(),
+                     v->blocksum.as<uint32_t>(), Int3{{g.og[0], g.og[1], g.og[2]}}, (uint32_t)p.max_voxels,
+                     (int4*)v->idx.p, (uint64_t*)nullptr, 0u, v->prefix.as<uint32_t>());
+  if (num_points) {
+    hipLaunchKernelGGL(k_vox_assign, dim3(ceil_div(num_points, 256)), dim3(256), 0, stream, v->pkey.as<uint32_t>(),
+                       num_points, v->bitmap.as<uint32_t>(), v->prefix.as<uint32_t>(), p.max_voxels,
+                       p.max_points_per_voxel, v->counts.as<uint32_t>(), v->mins.as<uint32_t>());
+    const uint32_t bound = (uint32_t)std::min<uint64_t>((uint64_t)p.max_voxels, num_points);
+    hipLaunchKernelGGL(k_vox_mean, dim3(ceil_div(bound * p.num_feature, 256)), dim3(256), 0, stream,
+                       (const _Float16*)points_fp16_dev, cnt, p.max_voxels, p.max_points_per_voxel, p.num_feature,
+                       v->counts.as<uint32_t>(), v->mins.as<uint32_t>(), (_Float16*)v->feats.p);
+  }
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
+const void* scn_voxelizer_features(const scn_voxelizer* v) { return v ? v->feats.p : nullptr; }
+const int32_t* scn_voxelizer_indices(const scn_voxelizer* v) { return v ? v->idx.as<int32_t>() : nullptr; }
+const uint32_t* scn_voxelizer_num_voxels_dev(const scn_voxelizer* v) { return v ? v->counters.as<uint32_t>() : nullptr; }
+const uint32_t* scn_voxelizer_points_per_voxel(const scn_voxelizer* v) { return v ? v->counts.as<uint32_t>() : nullptr; }
+
+uint32_t scn_voxelizer_num_voxels(scn_voxelizer* v, void* stream) {
+  if (!v) return 0;
+  if (hipMemcpyAsync(v->host_count, v->counters.p, 4, hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess) return 0;
+  if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return 0;
+  return *v->host_count;
+}
+
+void scn_voxelizer_grid_size(const scn_voxelizer* v, int order, int grid[3]) {
+  if (!v || !grid) return;
+  if (order == SCN_ORDER_ZYX) {
+    grid[0] = v->p.grid_size[2] + 1; grid[1] = v->p.grid_size[1]; grid[2] = v->p.grid_size[0];
+  } else {
+    grid[0] = v->p.grid_size[0]; grid[1] = v->p.grid_size[1]; grid[2] = v->p.grid_size[2] + 1;
+  }
+}
+
+// ---- rulebook -------------------------------------------------------------------------------
+struct scn_rulebook {
+  Rulebook rb;
+};
+
+scn_rulebook* scn_rulebook_create(uint32_t max_in, uint32_t max_out, int kernel_volume) {
+  if (kernel_volume <= 0 || (max_in == 0 && max_out == 0)) {
+    set_error("scn_rulebook_create: invalid arguments");
+    return nullptr;
+  }
+  auto* r = new scn_rulebook();
+  if (!r->rb.init(max_in, max_out, kernel_volume)) {
+    delete r;
+    return nullptr;
+  }
+  return r;
+}
+void scn_rulebook_destroy(scn_rulebook* rb) { delete rb; }
+
+int scn_rulebook_build_subm(scn_rulebook* rb, const int32_t* indices_dev, uint32_t n, const uint32_t* n_dev,
+                            const int grid[3], const int ksize[3], const int dilation[3], void* stream) {
+  SCN_REQUIRE(rb && grid && ksize && dilation && (indices_dev || n == 0), SCN_ERR_INVALID, "null pointer");
+  return rb->rb.build_subm(indices_dev, n, n_dev, grid, ksize, dilation, nullptr, (hipStream_t)stream);
+}
+int scn_rulebook_build_sparse(scn_rulebook* rb, const int32_t* indices_dev, uint32_t n, const uint32_t* n_dev,
+                              const int grid[3], const int ksize[3], const int stride[3], const int padding[3],
+                              const int dilation[3], void* stream) {
+  SCN_REQUIRE(rb && grid && ksize && stride && padding && dilation && (indices_dev || n == 0), SCN_ERR_INVALID,
+              "null pointer");
+  return rb->rb.build_sparse(indices_dev, n, n_dev, grid, ksize, stride, padding, dilation, nullptr,
+                             (hipStream_t)stream);
+}
+const int32_t* scn_rulebook_nbr(const scn_rulebook* rb) { return rb ? rb->rb.nbr.as<int32_t>() : nullptr; }
+uint32_t scn_rulebook_nbr_ld(const scn_rulebook* rb) { return rb ? rb->rb.ld : 0; }
+const int32_t* scn_rulebook_out_indices(const scn_rulebook* rb) { return rb ? rb->rb.out_indices : nullptr; }
+const uint32_t* scn_rulebook_num_out_dev(const scn_rulebook* rb) { return rb ? rb->rb.counters.as<uint32_t>() : nullptr; }
+const uint32_t* scn_rulebook_num_out_total_dev(const scn_rulebook* rb) {
+  return rb ? rb->rb.counters.as<uint32_t>() + 1 : nullptr;
+}
+void scn_rulebook_out_grid(const scn_rulebook* rb, int grid[3]) {
+  if (rb && grid)
+    for (int a = 0; a < 3; ++a) grid[a] = rb->rb.geom.grid_out[a];
+}
+int scn_rulebook_pairs(scn_rulebook* rb, int32_t* pair_in_dev, int32_t* pair_out_dev, int64_t* offsets_dev,
+                       uint64_t capacity, void* stream) {
+  SCN_REQUIRE(rb && pair_in_dev && pair_out_dev && offsets_dev, SCN_ERR_INVALID, "null pointer");
+  return rb->rb.pairs(pair_in_dev, pair_out_dev, offsets_dev, capacity, (hipStream_t)stream);
+}
+
+// ---- convolution ----------------------------------------------------------------------------
+struct scn_conv {
+  ConvWeights w;
+};
+
+scn_conv* scn_conv_create(const uint16_t* weight_fp16, const int weight_shape[5], const float* weight_dynamic_ranges,
+                          const uint16_t* bias_fp16, int precision) {
+  if (!weight_fp16 || !weight_shape || (precision != SCN_PRECISION_FP16 && precision != SCN_PRECISION_INT8)) {
+    set_error("scn_conv_create: invalid arguments");
+    return nullptr;
+  }
+  auto* c = new scn_conv();
+  if (!c->w.init(weight_fp16, weight_shape, weight_dynamic_ranges, bias_fp16, precision)) {
+    delete c;
+    return nullptr;
+  }
+  return c;
+}
+void scn_conv_destroy(scn_conv* c) { delete c; }
+
+int scn_conv_forward(const scn_conv* c, const scn_rulebook* rb, const scn_conv_io* io, void* stream) {
+  SCN_REQUIRE(c && rb && io, SCN_ERR_INVALID, "scn_conv_forward: null pointer");
+  SCN_REQUIRE(rb->rb.built, SCN_ERR_INVALID, "scn_conv_forward: rulebook not built");
+  SCN_REQUIRE(rb->rb.geom.kvol == c->w.kvol, SCN_ERR_INVALID, "scn_conv_forward: kernel volume mismatch (%d vs %d)",
+              rb->rb.geom.kvol, c->w.kvol);
+  return conv_forward(c->w, rb->rb.nbr.as<int32_t>(), rb->rb.ld, rb->rb.n_out_dev(), rb->rb.n_bound_out, *io,
+                      (hipStream_t)stream);
+}
+
+// ---- elementwise / dense --------------------------------------------------------------------
+int scn_convert_rows(const void* in_dev, int in_dtype, uint32_t in_c, uint32_t in_ld, float in_scale, void* out_dev,
+                     int out_dtype, uint32_t out_c, uint32_t out_ld, float out_scale, int relu, uint32_t n,
+                     const uint32_t* n_dev, void* stream) {
+  return convert_rows(in_dev, in_dtype, in_c, in_ld, in_scale, out_dev, out_dtype, out_c, out_ld, out_scale, relu, n,
+                      n_dev, (hipStream_t)stream);
+}
+int scn_add_relu(const void* a_dev, int a_dtype, float a_scale, float a_requant_scale, const void* b_dev, int b_dtype,
+                 float b_scale, float b_requant_scale, void* out_dev, int out_dtype, float out_scale, int relu,
+                 uint32_t c, uint32_t n, const uint32_t* n_dev, void* stream) {
+  return add_relu(a_dev, a_dtype, a_scale, a_requant_scale, b_dev, b_dtype, b_scale, b_requant_scale, out_dev,
+                  out_dtype, out_scale, relu, c, n, n_dev, (hipStream_t)stream);
+}
+int scn_scatter_dense(const void* feat_dev, int dtype, float scale, uint32_t c, uint32_t ld, const int32_t* indices_dev,
+                      uint32_t n, const uint32_t* n_dev, const int dense_shape[5], const int perm[5],
+                      void* out_fp16_dev, void* stream) {
+  return scatter_dense(feat_dev, dtype, scale, c, ld, indices_dev, n, n_dev, dense_shape, perm, out_fp16_dev,
+                       (hipStream_t)stream);
+}
+
+}  // extern "C"

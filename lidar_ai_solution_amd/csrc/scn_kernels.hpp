@@ -1,0 +1,103 @@
+// Internal C++ interface between the kernel translation unit and the engine / C-ABI layers.
+#pragma once
+
+#include "scn_common.hpp"
+
+namespace scn {
+
+// Open-addressing coordinate hash: 64-bit slots {key (linear voxel index) << 32 | row}.
+constexpr uint64_t kEmptySlot = ~0ull;
+
+struct CoordTable {
+  DevBuf buf;
+  size_t cap = 0;     // allocated slots, power of two
+  uint32_t mask = 0;  // slots in use - 1 (power of two <= cap), set by the last build
+  bool alloc_for(uint32_t max_rows);
+  uint64_t* slots() const { return buf.as<uint64_t>(); }
+};
+
+size_t hash_capacity_for(uint32_t n);
+
+struct ConvGeom {
+  int grid_in[3];
+  int grid_out[3];
+  int ks[3];
+  int stride[3];
+  int pad[3];
+  int dil[3];
+  int kvol;
+};
+
+// Rulebook object (= scn_rulebook of the C ABI).
+struct Rulebook {
+  uint32_t max_in = 0, max_out = 0;
+  int kvol_cap = 0;
+  bool subm = false;
+  ConvGeom geom{};
+  CoordTable own_in_table;    // hash of the input rows when no shared table is passed
+  CoordTable out_table;       // strided only: hash of the output rows (next stage's lookups)
+  const CoordTable* in_table = nullptr;  // the table actually used for input lookups
+  DevBuf nbr;                 // int32 [kvol_cap][ld]
+  uint32_t ld = 0;
+  DevBuf out_idx;             // int32 [max_out][4] (strided)
+  DevBuf counters;            // uint32: [0] n_out kept, [1] n_out before truncation, [2..] scratch
+  DevBuf bitmap, blocksum;    // strided: occupancy bitmap of the output grid + per-block popcounts
+  size_t bitmap_words = 0;
+  DevBuf pair_scratch;        // pair compaction: per (k, block) counts
+  const int32_t* in_indices = nullptr;
+  const int32_t* out_indices = nullptr;  // subm: aliases in_indices
+  uint32_t n_bound_in = 0, n_bound_out = 0;
+  bool built = false;
+
+  bool init(uint32_t max_in_, uint32_t max_out_, int kvol);
+  int build_subm(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3], const int ks[3],
+                 const int dil[3], const CoordTable* shared_in_table, hipStream_t stream);
+  int build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3], const int ks[3],
+                   const int stride[3], const int pad[3], const int dil[3], const CoordTable* shared_in_table,
+                   hipStream_t stream);
+  int pairs(int32_t* pair_in, int32_t* pair_out, int64_t* offsets, uint64_t capacity, hipStream_t stream);
+  const uint32_t* n_out_dev() const { return counters.as<uint32_t>(); }
+};
+
+// Packed weights of one convolution (= scn_conv of the C ABI).
+struct ConvWeights {
+  int cin = 0, cout = 0, kvol = 0, ks[3] = {1, 1, 1};
+  int precision = SCN_PRECISION_FP16;  // compute precision
+  int chunks = 0;   // 16-byte chunks per (padded) input row
+  int mtiles = 0;   // ceil(cout / 16)
+  int steps = 0;    // MFMA K-steps = ceil(kvol * chunks / 4)
+  uint32_t cin_pad = 0;  // padded input channels the kernel expects (elements)
+  DevBuf wfrag;     // [steps][mtiles][64] x 16 bytes, MFMA A-operand order
+  DevBuf wscale;    // fp32 [cout_pad]: s_w[c] (int8) or 1
+  DevBuf bias;      // fp32 [cout_pad]
+  bool init(const uint16_t* w_fp16, const int shape[5], const float* ranges, const uint16_t* bias_fp16, int prec);
+};
+
+int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, const uint32_t* n_out_dev,
+                 uint32_t n_bound, const scn_conv_io& io, hipStream_t stream);
+
+int fill_u32(void* p, uint32_t value, size_t count, hipStream_t stream);
+int hash_build(const CoordTable& t, const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3],
+               uint32_t* n_eff_out, hipStream_t stream);
+int hash_query(const CoordTable& t, const int32_t* coords, uint32_t n, const int grid[3], int32_t* rows,
+               hipStream_t stream);
+
+int convert_rows(const void* in, int in_dtype, uint32_t in_c, uint32_t in_ld, float in_scale, void* out,
+                 int out_dtype, uint32_t out_c, uint32_t out_ld, float out_scale, int relu, uint32_t n,
+                 const uint32_t* n_dev, hipStream_t stream);
+int add_relu(const void* a, int a_dtype, float a_scale, float a_rq, const void* b, int b_dtype, float b_scale,
+             float b_rq, void* out, int out_dtype, float out_scale, int relu, uint32_t c, uint32_t n,
+             const uint32_t* n_dev, hipStream_t stream);
+int scatter_dense(const void* feat, int dtype, float scale, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
+                  const uint32_t* n_dev, const int dense_shape[5], const int perm[5], void* out, hipStream_t stream);
+
+}  // namespace scn
+
+// Voxelizer object of the C ABI.
+struct scn_voxelizer {
+  scn_voxelization_param p{};
+  scn::DevBuf bitmap, prefix, blocksum, pkey, mins, counts, feats, idx, counters;
+  size_t words = 0;
+  uint32_t* host_count = nullptr;  // pinned
+  int last_order = SCN_ORDER_XYZ;
+};

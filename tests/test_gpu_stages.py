@@ -1,0 +1,410 @@
+"""Parity of every HIP stage with the CPU oracle, through the C ABI.  Needs a MI355X."""
+import ctypes as C
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from lidar_ai_solution_amd import capi, synth
+from oracle import scn_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+from tests.gpu_helpers import DEV, GpuConv, GpuRulebook, copy_from_ptr, i3, ptr, read_u32, stream, to_dev  # noqa: E402
+
+KNOWN = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "known_answers.json")))
+
+
+def note(msg):
+    print(f"[case] {msg}", flush=True)
+
+
+# ----------------------------------------------------------------------------- hash
+def test_hash_build_and_query(centerpoint_input):
+    note("hash build/query on the 79,745-voxel fixture")
+    L = capi.lib()
+    _, idx = centerpoint_input
+    assert L.scn_hash_u64(85017599) == O.hash64(85017599)
+    n = idx.shape[0]
+    cap = L.scn_hash_capacity_for(n)
+    assert cap >= 2 * n and cap & (cap - 1) == 0
+    table = torch.zeros(cap, dtype=torch.int64, device=DEV)
+    d_idx = to_dev(idx)
+    grid = (41, 1440, 1440)
+    capi.check(L.scn_hash_build(ptr(table), cap, ptr(d_idx), n, None, i3(grid), stream()))
+    rng = np.random.default_rng(0)
+    q = idx[rng.permutation(n)[:5000]].copy()
+    miss = q.copy()
+    miss[:, 3] = (miss[:, 3] + 1) % 1440
+    d = {tuple(r): i for i, r in enumerate(idx)}
+    qq = np.concatenate([q, miss])
+    rows = torch.zeros(qq.shape[0], dtype=torch.int32, device=DEV)
+    d_qq = to_dev(qq)
+    capi.check(L.scn_hash_query(ptr(table), cap, ptr(d_qq), qq.shape[0], i3(grid), ptr(rows), stream()))
+    torch.cuda.synchronize()
+    want = np.array([d.get(tuple(r), -1) for r in qq], np.int32)
+    assert np.array_equal(rows.cpu().numpy(), want)
+    # occupancy: every row landed in exactly one slot
+    t = table.cpu().numpy().view(np.uint64)
+    used = t != np.uint64(0xFFFFFFFFFFFFFFFF)
+    assert int(used.sum()) == n
+    assert np.array_equal(np.sort((t[used] & np.uint64(0xFFFFFFFF)).astype(np.int64)), np.arange(n))
+
+
+# ----------------------------------------------------------------------------- rulebooks
+STAGES = [((3, 3, 3), (2, 2, 2), (1, 1, 1)), ((3, 3, 3), (2, 2, 2), (1, 1, 1)),
+          ((3, 3, 3), (2, 2, 2), (0, 1, 1)), ((3, 1, 1), (2, 1, 1), (0, 0, 0))]
+
+
+def _check_pairs(rb_gpu, ref):
+    pin, pout, offs = rb_gpu.pairs(max(ref.num_pairs, 1))
+    assert np.array_equal(offs, ref.offsets)
+    assert np.array_equal(pout, ref.pair_out)
+    assert np.array_equal(pin, ref.pair_in)
+
+
+def test_rulebooks_on_reference_fixture_all_stages(centerpoint_input):
+    _, idx = centerpoint_input
+    ka = KNOWN["centerpoint_fixture"]
+    grid = [41, 1440, 1440]
+    for s in range(4):
+        n = idx.shape[0]
+        note(f"rulebooks stage {s}: n={n} grid={grid}")
+        d_idx = to_dev(idx)
+        sub = GpuRulebook(n, n, 27)
+        sub.build_subm(d_idx, n, grid, (3, 3, 3))
+        ref = O.rulebook_subm(idx, grid, (3, 3, 3))
+        assert ref.num_pairs == ka["subm_pairs"][s]
+        _check_pairs(sub, ref)
+        k, st, p = STAGES[s]
+        sp = GpuRulebook(n, 200000, int(np.prod(k)))
+        sp.build_sparse(d_idx, n, grid, k, st, p)
+        ref2 = O.rulebook_sparse(idx, grid, k, st, p)
+        assert sp.out_grid() == ref2.out_grid == ka["grids"][s + 1]
+        assert sp.n_out() == ref2.n_out == ka["active"][s + 1]
+        assert np.array_equal(sp.out_indices(), ref2.out_indices)
+        _check_pairs(sp, ref2)
+        idx, grid = ref2.out_indices, ref2.out_grid
+
+
+def test_sparse_rulebook_truncation_empty_and_device_count():
+    rng = np.random.default_rng(11)
+    grid = (9, 40, 37)
+    vol = int(np.prod(grid))
+    lin = rng.choice(vol, 3000, replace=False)
+    idx = np.zeros((3000, 4), np.int32)
+    idx[:, 3] = lin % grid[2]; idx[:, 2] = (lin // grid[2]) % grid[1]; idx[:, 1] = lin // (grid[2] * grid[1])
+    d_idx = to_dev(idx)
+    note("sparse rulebook truncated to 500 outputs")
+    rb = GpuRulebook(3000, 500, 27)
+    rb.build_sparse(d_idx, 3000, grid, (3, 3, 3), (2, 2, 2), (1, 1, 1))
+    ref = O.rulebook_sparse(idx, grid, (3, 3, 3), (2, 2, 2), (1, 1, 1), max_out=500)
+    assert rb.n_out() == 500 and rb.n_out_total() == ref.n_out_total
+    assert np.array_equal(rb.out_indices(), ref.out_indices)
+    _check_pairs(rb, ref)
+    note("device-side row count smaller than the bound")
+    n_dev = torch.tensor([1234], dtype=torch.int32, device=DEV)
+    rb2 = GpuRulebook(3000, 3000, 27)
+    rb2.build_sparse(d_idx, 3000, grid, (3, 3, 3), (2, 2, 2), (1, 1, 1), n_dev=n_dev)
+    ref2 = O.rulebook_sparse(idx[:1234], grid, (3, 3, 3), (2, 2, 2), (1, 1, 1))
+    assert rb2.n_out() == ref2.n_out
+    assert np.array_equal(rb2.out_indices(), ref2.out_indices)
+    _check_pairs(rb2, ref2)
+    sub = GpuRulebook(3000, 3000, 27)
+    sub.build_subm(d_idx, 3000, grid, (3, 3, 3), n_dev=n_dev)
+    _check_pairs(sub, O.rulebook_subm(idx[:1234], grid, (3, 3, 3)))
+    note("empty input")
+    n0 = torch.tensor([0], dtype=torch.int32, device=DEV)
+    rb3 = GpuRulebook(3000, 3000, 27)
+    rb3.build_sparse(d_idx, 3000, grid, (3, 3, 3), (2, 2, 2), (1, 1, 1), n_dev=n0)
+    assert rb3.n_out() == 0
+    pin, pout, offs = rb3.pairs(16)
+    assert offs[-1] == 0
+    note("dilated and non-cubic kernels")
+    for ks, st, pd, dl in [((3, 3, 3), (1, 1, 1), (2, 2, 2), (2, 2, 2)), ((1, 3, 3), (1, 2, 2), (0, 1, 1), (1, 1, 1)),
+                           ((2, 2, 2), (2, 2, 2), (0, 0, 0), (1, 1, 1)), ((1, 1, 3), (1, 1, 2), (0, 0, 0), (1, 1, 1))]:
+        r = GpuRulebook(3000, 3000 * 8, int(np.prod(ks)))
+        r.build_sparse(d_idx, 3000, grid, ks, st, pd, dl)
+        rr = O.rulebook_sparse(idx, grid, ks, st, pd, dl)
+        assert r.n_out() == rr.n_out and np.array_equal(r.out_indices(), rr.out_indices)
+        _check_pairs(r, rr)
+    s2 = GpuRulebook(3000, 3000, 27)
+    s2.build_subm(d_idx, 3000, grid, (3, 3, 3), (2, 2, 2))
+    _check_pairs(s2, O.rulebook_subm(idx, grid, (3, 3, 3), (2, 2, 2)))
+
+
+# ----------------------------------------------------------------------------- convolution
+def _weights(rng, cout, ks, cin, std=0.02):
+    w = (rng.standard_normal((cout, *ks, cin)) * std).astype(np.float16)
+    b = (rng.standard_normal(cout) * std).astype(np.float16)
+    ranges = np.abs(w.astype(np.float32)).reshape(cout, -1).max(1)
+    return w, b, ranges
+
+
+def test_config1_single_int8_subm_layer():
+    """One int8 SubMConv3d 3x3x3 16->16 on 20,000 uniform voxels: int32 accumulators and the int8
+    requantised ReLU output are bit-exact."""
+    note("config 1: int8 subm 16->16, 20000 voxels")
+    rng = np.random.default_rng(0)
+    grid = (41, 1440, 1440)
+    idx = synth.uniform_voxels(0, 20000, grid)
+    x = rng.integers(-127, 128, (20000, 16)).astype(np.int8)
+    w, b, ranges = _weights(rng, 16, (3, 3, 3), 16)
+    s_x = 0.05
+    ref_rb = O.rulebook_subm(idx, grid, (3, 3, 3))
+    wq, s_w = O.quantize_weights(w, ranges)
+    acc_ref = O.conv_int8_acc(x, wq, ref_rb)
+    scale = (np.float32(s_x) * s_w).astype(np.float32)
+    y = np.maximum(acc_ref.astype(np.float32) * scale + b.astype(np.float32), 0)
+    s_out = float(np.float32(np.percentile(y, 99.99)) / np.float32(127))
+    out_ref = O.epilogue(acc_ref, scale, b.astype(np.float32), True, True, s_out)
+    rb = GpuRulebook(20000, 20000, 27)
+    rb.build_subm(to_dev(idx), 20000, grid, (3, 3, 3))
+    conv = GpuConv(w, ranges, b, capi.PRECISION_INT8)
+    out, acc = conv.forward(rb, to_dev(x), 20000, x_scale=s_x, relu=True, out_int8=True, out_scale=s_out, want_acc=True)
+    assert np.array_equal(acc.cpu().numpy(), acc_ref)
+    assert np.array_equal(out.cpu().numpy(), out_ref)
+    assert ref_rb.num_pairs >= 20000 and np.abs(out_ref).max() > 20
+
+
+SHAPES = [(16, 16), (16, 32), (32, 32), (32, 64), (64, 64), (64, 128), (128, 128)]
+
+
+@pytest.mark.parametrize("cin,cout", SHAPES)
+def test_int8_conv_shapes_bit_exact(cin, cout, centerpoint_input):
+    _, idx_all = centerpoint_input
+    rng = np.random.default_rng(cin * 1000 + cout)
+    idx = idx_all[:30000]
+    n = idx.shape[0]
+    grid = (41, 1440, 1440)
+    subm = cin == cout
+    note(f"int8 conv {cin}->{cout} {'subm' if subm else 'strided'} on {n} fixture voxels")
+    x = rng.integers(-127, 128, (n, cin)).astype(np.int8)
+    w, b, ranges = _weights(rng, cout, (3, 3, 3), cin)
+    s_x, s_out = 0.031, 0.043
+    if subm:
+        ref_rb = O.rulebook_subm(idx, grid, (3, 3, 3))
+        rb = GpuRulebook(n, n, 27)
+        rb.build_subm(to_dev(idx), n, grid, (3, 3, 3))
+    else:
+        ref_rb = O.rulebook_sparse(idx, grid, (3, 3, 3), (2, 2, 2), (1, 1, 1))
+        rb = GpuRulebook(n, 200000, 27)
+        rb.build_sparse(to_dev(idx), n, grid, (3, 3, 3), (2, 2, 2), (1, 1, 1))
+    wq, s_w = O.quantize_weights(w, ranges)
+    acc_ref = O.conv_int8_acc(x, wq, ref_rb)
+    scale = (np.float32(s_x) * s_w).astype(np.float32)
+    conv = GpuConv(w, ranges, b, capi.PRECISION_INT8)
+    out, acc = conv.forward(rb, to_dev(x), ref_rb.n_out, x_scale=s_x, relu=True, out_int8=True, out_scale=s_out, want_acc=True)
+    assert np.array_equal(acc.cpu().numpy(), acc_ref)
+    assert np.array_equal(out.cpu().numpy(), O.epilogue(acc_ref, scale, b.astype(np.float32), True, True, s_out))
+    out16, _ = conv.forward(rb, to_dev(x), ref_rb.n_out, x_scale=s_x, relu=False, out_int8=False)
+    ref16 = O.epilogue(acc_ref, scale, b.astype(np.float32), False, False)
+    assert np.array_equal(out16.cpu().numpy().view(np.uint16), ref16.view(np.uint16))
+
+
+@pytest.mark.parametrize("cin,cout", [(5, 16), (16, 16), (32, 64), (128, 128)])
+def test_fp16_conv_within_tolerance(cin, cout, centerpoint_input):
+    """fp16 MFMA path: fp32 accumulation in hardware order.  Tolerance (stated): every accumulator
+    within 2e-3 * (sum of |products|) + 1e-6 of the fp32 oracle; fp16 outputs within 1 ulp-ish
+    (rtol 2e-3, atol 1e-3)."""
+    feats, idx_all = centerpoint_input
+    rng = np.random.default_rng(cin * 7 + cout)
+    idx = idx_all[:30000]
+    n = idx.shape[0]
+    grid = (41, 1440, 1440)
+    note(f"fp16 conv {cin}->{cout} on {n} fixture voxels")
+    if cin == 5:
+        x = feats[:n].astype(np.float16)
+    else:
+        x = rng.standard_normal((n, cin)).astype(np.float16)
+    w, b, _ = _weights(rng, cout, (3, 3, 3), cin, std=0.05)
+    ref_rb = O.rulebook_subm(idx, grid, (3, 3, 3))
+    wf = np.ascontiguousarray(w.astype(np.float32).reshape(cout, 27, cin).transpose(1, 0, 2))
+    acc_ref = O.conv_f32_acc(x.astype(np.float32), wf, ref_rb)
+    mag = O.conv_f32_acc(np.abs(x.astype(np.float32)), np.abs(wf), ref_rb)
+    rb = GpuRulebook(n, n, 27)
+    rb.build_subm(to_dev(idx), n, grid, (3, 3, 3))
+    conv = GpuConv(w, None, b, capi.PRECISION_FP16)
+    cpad = 8 if cin == 5 else cin
+    xp = np.zeros((n, cpad), np.float16)
+    xp[:, :cin] = x
+    out, acc = conv.forward(rb, to_dev(xp), n, relu=True, want_acc=True)
+    acc = acc.cpu().numpy()
+    assert np.all(np.abs(acc - acc_ref) <= 2e-3 * mag + 1e-6)
+    ref = O.epilogue(acc_ref, None, b.astype(np.float32), True, False).astype(np.float32)
+    assert np.allclose(out.cpu().numpy().astype(np.float32), ref, rtol=2e-3, atol=1e-3)
+
+
+def test_fused_residual_epilogue_matches_unfused_oracle(centerpoint_input):
+    """conv2 -> Add(identity) -> ReLU fused into one kernel equals the node-by-node oracle."""
+    _, idx_all = centerpoint_input
+    rng = np.random.default_rng(21)
+    idx = idx_all[:20000]
+    n = idx.shape[0]
+    grid = (41, 1440, 1440)
+    cin = cout = 32
+    x = rng.integers(-127, 128, (n, cin)).astype(np.int8)
+    ident = rng.integers(0, 128, (n, cout)).astype(np.int8)
+    w, b, ranges = _weights(rng, cout, (3, 3, 3), cin)
+    s_x, s_mid, s_res, s_out = 0.02, 0.035, 0.027, 0.05
+    ref_rb = O.rulebook_subm(idx, grid, (3, 3, 3))
+    wq, s_w = O.quantize_weights(w, ranges)
+    acc_ref = O.conv_int8_acc(x, wq, ref_rb)
+    scale = (np.float32(s_x) * s_w).astype(np.float32)
+    rb = GpuRulebook(n, n, 27)
+    rb.build_subm(to_dev(idx), n, grid, (3, 3, 3))
+    conv = GpuConv(w, ranges, b, capi.PRECISION_INT8)
+    note("int8 conv -> int8 add -> relu")
+    mid = O.epilogue(acc_ref, scale, b.astype(np.float32), False, True, s_mid)
+    want = O.add(mid, s_mid, ident, s_res, True, True, s_out)
+    out, _ = conv.forward(rb, to_dev(x), n, x_scale=s_x, relu=False, out_int8=True, out_scale=s_out,
+                          res=to_dev(ident), res_scale=s_res, mid_int8=True, mid_scale=s_mid, relu2=True)
+    assert np.array_equal(out.cpu().numpy(), want)
+    note("fp16-stored conv output and fp16 identity, int8 add re-quantising both, int8 out")
+    ident16 = (rng.standard_normal((n, cout)) * 2).astype(np.float16)
+    mid16 = O.epilogue(acc_ref, scale, b.astype(np.float32), False, False)
+    s_add = 0.04
+    want2 = O.add(O.quantize(mid16, s_add), s_add, O.quantize(ident16, s_add), s_add, True, True, s_out)
+    out2, _ = conv.forward(rb, to_dev(x), n, x_scale=s_x, relu=False, out_int8=True, out_scale=s_out,
+                           res=to_dev(ident16), mid_int8=False, a_rq=s_add, b_rq=s_add, relu2=True)
+    assert np.array_equal(out2.cpu().numpy(), want2)
+    note("fp16 add of fp16 operands, fp16 out")
+    want3 = O.add(mid16, 1.0, ident16, 1.0, True, False)
+    out3, _ = conv.forward(rb, to_dev(x), n, x_scale=s_x, relu=False, out_int8=False,
+                           res=to_dev(ident16), mid_int8=False, relu2=True)
+    assert np.array_equal(out3.cpu().numpy().view(np.uint16), want3.view(np.uint16))
+
+
+# ----------------------------------------------------------------------------- elementwise / dense
+def test_convert_add_and_dense():
+    L = capi.lib()
+    rng = np.random.default_rng(31)
+    n, c = 5000, 32
+    note("quantise / dequantise / pad rows")
+    x = (rng.standard_normal((n, 5)) * 20).astype(np.float16)
+    s = 0.3
+    out = torch.zeros((n, 16), dtype=torch.int8, device=DEV)
+    d_x = to_dev(x)
+    capi.check(L.scn_convert_rows(ptr(d_x), capi.DTYPE_FP16, 5, 5, 1.0, ptr(out), capi.DTYPE_INT8, 16, 16, s, 0, n, None, stream()))
+    torch.cuda.synchronize()
+    want = np.zeros((n, 16), np.int8)
+    want[:, :5] = O.quantize(x, s)
+    assert np.array_equal(out.cpu().numpy(), want)
+    q = rng.integers(-127, 128, (n, c)).astype(np.int8)
+    out = torch.zeros((n, c), dtype=torch.float16, device=DEV)
+    d_q = to_dev(q)
+    capi.check(L.scn_convert_rows(ptr(d_q), capi.DTYPE_INT8, c, c, s, ptr(out), capi.DTYPE_FP16, c, c, 1.0, 0, n, None, stream()))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), O.dequantize(q, s).view(np.uint16))
+    padded = torch.full((n, 8), 7, dtype=torch.float16, device=DEV)
+    capi.check(L.scn_convert_rows(ptr(d_x), capi.DTYPE_FP16, 5, 5, 1.0, ptr(padded), capi.DTYPE_FP16, 8, 8, 1.0, 0, n, None, stream()))
+    torch.cuda.synchronize()
+    pw = np.zeros((n, 8), np.float16); pw[:, :5] = x
+    assert np.array_equal(padded.cpu().numpy().view(np.uint16), pw.view(np.uint16))
+    note("add + relu, int8 and fp16 operands, device-side count")
+    a = rng.integers(-127, 128, (n, c)).astype(np.int8)
+    b = rng.integers(-127, 128, (n, c)).astype(np.int8)
+    n_dev = torch.tensor([4321], dtype=torch.int32, device=DEV)
+    out = torch.zeros((n, c), dtype=torch.int8, device=DEV)
+    da, db = to_dev(a), to_dev(b)  # keep both alive: the caching allocator would hand b the memory of a
+    capi.check(L.scn_add_relu(ptr(da), capi.DTYPE_INT8, 0.03, 0.0, ptr(db), capi.DTYPE_INT8, 0.02, 0.0, ptr(out),
+                              capi.DTYPE_INT8, 0.04, 1, c, n, ptr(n_dev), stream()))
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert np.array_equal(got[:4321], O.add(a[:4321], 0.03, b[:4321], 0.02, True, True, 0.04)) and not got[4321:].any()
+    h1 = rng.standard_normal((n, c)).astype(np.float16); h2 = rng.standard_normal((n, c)).astype(np.float16)
+    out = torch.zeros((n, c), dtype=torch.float16, device=DEV)
+    d1, d2 = to_dev(h1), to_dev(h2)
+    capi.check(L.scn_add_relu(ptr(d1), capi.DTYPE_FP16, 1.0, 0.0, ptr(d2), capi.DTYPE_FP16, 1.0, 0.0, ptr(out),
+                              capi.DTYPE_FP16, 1.0, 0, c, n, None, stream()))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), O.add(h1, 1.0, h2, 1.0, False, False).view(np.uint16))
+    note("scatter dense, plain and with the fused transpose")
+    dims = (2, 45, 37)
+    lin = rng.choice(int(np.prod(dims)), 1500, replace=False)
+    idx = np.zeros((1500, 4), np.int32)
+    idx[:, 3] = lin % dims[2]; idx[:, 2] = (lin // dims[2]) % dims[1]; idx[:, 1] = lin // (dims[2] * dims[1])
+    feat = rng.standard_normal((1500, 16)).astype(np.float16)
+    dense_ref = O.scatter_dense(feat, idx, dims)
+    shape = capi.i5(1, 16, *dims)
+    out = torch.full((1, 16, *dims), 3, dtype=torch.float16, device=DEV)
+    d_feat, d_idx = to_dev(feat), to_dev(idx)
+    capi.check(L.scn_scatter_dense(ptr(d_feat), capi.DTYPE_FP16, 1.0, 16, 16, ptr(d_idx), 1500, None, shape, None, ptr(out), stream()))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), dense_ref.view(np.uint16))
+    perm = (0, 1, 4, 2, 3)
+    out = torch.full((1, 16, dims[2], dims[0], dims[1]), 3, dtype=torch.float16, device=DEV)
+    capi.check(L.scn_scatter_dense(ptr(d_feat), capi.DTYPE_FP16, 1.0, 16, 16, ptr(d_idx), 1500, None, shape,
+                                   capi.i5(*perm), ptr(out), stream()))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), np.ascontiguousarray(dense_ref.transpose(perm)).view(np.uint16))
+    qf = rng.integers(-127, 128, (1500, 16)).astype(np.int8)
+    out = torch.zeros((1, 16, *dims), dtype=torch.float16, device=DEV)
+    d_qf = to_dev(qf)
+    capi.check(L.scn_scatter_dense(ptr(d_qf), capi.DTYPE_INT8, 0.05, 16, 16, ptr(d_idx), 1500, None, shape, None, ptr(out), stream()))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), O.scatter_dense(O.dequantize(qf, 0.05), idx, dims).view(np.uint16))
+
+
+# ----------------------------------------------------------------------------- voxelization
+def _voxelizer(max_voxels=160000, max_points=300000):
+    p = capi.VoxelizationParam()
+    p.min_range[:] = synth.MIN_RANGE; p.max_range[:] = synth.MAX_RANGE; p.voxel_size[:] = synth.VOXEL_SIZE
+    p.grid_size[:] = synth.GRID_XYZ
+    p.num_feature, p.max_voxels, p.max_points_per_voxel, p.max_points = 5, max_voxels, 10, max_points
+    h = capi.lib().scn_voxelizer_create(C.byref(p))
+    assert h
+    return h
+
+
+def _run_voxelizer(h, pts, order, max_voxels):
+    L = capi.lib()
+    code = capi.ORDER_ZYX if order == "zyx" else capi.ORDER_XYZ
+    d = to_dev(pts)
+    capi.check(L.scn_voxelizer_forward(h, ptr(d), pts.shape[0], code, stream()))
+    nv = L.scn_voxelizer_num_voxels(h, stream())
+    f = copy_from_ptr(L.scn_voxelizer_features(h), (nv, 5), np.float16).cpu().numpy()
+    i = copy_from_ptr(L.scn_voxelizer_indices(h), (nv, 4), np.int32).cpu().numpy()
+    c = copy_from_ptr(L.scn_voxelizer_points_per_voxel(h), (nv,), np.int32).cpu().numpy()
+    return f, i, c
+
+
+@pytest.mark.parametrize("order", ["zyx", "xyz"])
+def test_voxelization_real_frame_bit_exact(order, nuscenes_frame):
+    note(f"voxelization of the 271,156-point frame, order {order}")
+    L = capi.lib()
+    h = _voxelizer()
+    try:
+        f, i, c = _run_voxelizer(h, nuscenes_frame, order, 160000)
+        rf, ri, rc = O.voxelize(nuscenes_frame, synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, order=order)
+        assert f.shape[0] == KNOWN["nuscenes_frame"]["voxels"]
+        assert np.array_equal(i, ri) and np.array_equal(c, rc)
+        assert np.array_equal(f.view(np.uint16), rf.view(np.uint16))
+        g = capi.i3()
+        L.scn_voxelizer_grid_size(h, capi.ORDER_ZYX if order == "zyx" else capi.ORDER_XYZ, g)
+        assert list(g) == ([41, 1440, 1440] if order == "zyx" else [1440, 1440, 41])
+        note("second frame on the same object (state is cleared), then an empty frame")
+        pts2 = synth.lidar_frame(3, 100000)
+        f2, i2, c2 = _run_voxelizer(h, pts2, order, 160000)
+        rf2, ri2, rc2 = O.voxelize(pts2, synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, order=order)
+        assert np.array_equal(i2, ri2) and np.array_equal(c2, rc2) and np.array_equal(f2.view(np.uint16), rf2.view(np.uint16))
+        f0, i0, _ = _run_voxelizer(h, pts2[:0], order, 160000)
+        assert f0.shape[0] == 0
+    finally:
+        L.scn_voxelizer_destroy(h)
+
+
+def test_voxelization_truncates_at_max_voxels(nuscenes_frame):
+    note("voxelization with max_voxels=5000")
+    L = capi.lib()
+    h = _voxelizer(max_voxels=5000)
+    try:
+        f, i, c = _run_voxelizer(h, nuscenes_frame[:60000], "zyx", 5000)
+        rf, ri, rc = O.voxelize(nuscenes_frame[:60000], synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ,
+                                max_voxels=5000, order="zyx")
+        assert f.shape[0] == 5000 and np.array_equal(i, ri) and np.array_equal(c, rc)
+        assert np.array_equal(f.view(np.uint16), rf.view(np.uint16))
+    finally:
+        L.scn_voxelizer_destroy(h)
