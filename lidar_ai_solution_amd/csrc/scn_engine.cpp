@@ -1,0 +1,1514 @@
+// Graph builder, precision planner and executor of the SCN engine, plus the ONNX loader.
+//
+// Mirrors the builder / engine surface of the reference
+// (libraries/3DSparseConvolution/libspconv/include/spconv/engine.hpp:38-167) behind the C ABI and
+// what its loader does with a model file (libraries/3DSparseConvolution/src/onnx-parser.cpp:101-231).
+//
+// Execution model: build() turns the node list into a flat list of steps (hash build, rulebook
+// build, conversion, convolution with fused epilogue, add, relu, dense scatter).  forward() only
+// enqueues kernels on the caller's stream: row counts live in device memory, launch sizes come from
+// host-side bounds, nothing is allocated after the first call with a given grid size.
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <fstream>
+#include <functional>
+#include <map>
+#include <memory>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "scn_kernels.hpp"
+
+namespace scn {
+
+enum class Op { Conv, Add, Relu, Dense, Reshape, Transpose };
+
+static const char* op_name(Op op) {
+  switch (op) {
+    case Op::Conv: return "SparseConvolution";
+    case Op::Add: return "Add";
+    case Op::Relu: return "Relu";
+    case Op::Dense: return "ScatterDense";
+    case Op::Reshape: return "Reshape";
+    case Op::Transpose: return "Transpose";
+  }
+  return "?";
+}
+
+struct NodeDesc {
+  Op op;
+  std::string name;
+  std::vector<int> in;
+  int out = -1;
+  // conv
+  std::vector<uint16_t> weight;
+  int wshape[5] = {0, 0, 0, 0, 0};
+  std::vector<float> wranges;
+  std::vector<uint16_t> bias;
+  std::string activation;
+  int ks[3] = {1, 1, 1}, stride[3] = {1, 1, 1}, pad[3] = {0, 0, 0}, dil[3] = {1, 1, 1};
+  float in_range = 0.f;
+  bool subm = false;
+  uint32_t max_out = 150000;
+  std::string rulebook;
+  int precision = SCN_PRECISION_FP16, out_precision = SCN_PRECISION_FP16;
+  // add
+  float a_range = 0.f, b_range = 0.f;
+  // dense
+  std::string format;
+  int in_spatial[3] = {0, 0, 0};
+  std::vector<int> out_shape;
+  float dense_range = 0.f;
+  // reshape / transpose
+  std::vector<int64_t> dims;
+};
+
+struct TensorDesc {
+  std::string name;
+  int producer = -1;  // node index, -1 for graph inputs
+};
+
+}  // namespace scn
+
+using namespace scn;
+
+struct scn_builder {
+  std::vector<TensorDesc> tensors;
+  std::vector<NodeDesc> nodes;
+  std::vector<int> inputs, outputs;
+  int new_tensor(const char* name, int producer) {
+    TensorDesc t;
+    t.name = name ? name : "";
+    t.producer = producer;
+    tensors.push_back(t);
+    return (int)tensors.size() - 1;
+  }
+  bool valid_tensor(int t) const { return t >= 0 && t < (int)tensors.size(); }
+};
+
+namespace scn {
+
+// ---------------------------------------------------------------------------------------------
+// runtime objects
+// ---------------------------------------------------------------------------------------------
+struct CoordSet {
+  const int32_t* idx = nullptr;
+  const uint32_t* n_dev = nullptr;
+  uint32_t n_bound = 0;  // host-side bound of the row count for the current forward
+  uint32_t cap = 0;      // allocated rows
+  int grid[3] = {0, 0, 0};
+  const CoordTable* table = nullptr;  // hash of these coordinates (set once built in this forward)
+  CoordTable own_table;               // only for graph inputs
+  int producer_rulebook = -1;         // strided rulebook that creates this set (-1: graph input)
+};
+
+struct RtTensor {
+  bool dense = false;
+  int dtype = SCN_DTYPE_FP16;
+  float scale = 1.f;   // int8: value = q * scale
+  int c = 0;           // logical channels
+  uint32_t ld = 0;     // row stride in elements
+  int coord = -1;      // CoordSet index (sparse)
+  DevBuf buf;          // owned storage (not for graph inputs / views)
+  void* data = nullptr;
+  DevBuf acc;          // raw accumulators (keep-all mode)
+  std::vector<int64_t> shape;  // dense
+  int view_of = -1;    // dense view of another tensor (reshape / fused transpose)
+  bool materialised = false;  // false: fused away, never written
+};
+
+enum class StepKind { InputCount, HashBuild, RulebookSubm, RulebookSparse, Convert, Conv, Add, Relu, Dense };
+
+struct Step {
+  StepKind kind;
+  int node = -1;       // graph node this step belongs to (for profiling names)
+  std::string label;
+  // generic operands
+  int t_in = -1, t_in2 = -1, t_out = -1;
+  int coord = -1, coord_out = -1;
+  int rulebook = -1;
+  int conv = -1;
+  // convert
+  int cv_dtype = 0;
+  float cv_scale = 1.f;
+  uint32_t cv_c = 0;
+  int relu = 0;
+  // conv epilogue
+  float x_scale = 1.f;
+  bool fused_add = false;
+  int mid_dtype = 0;
+  float mid_scale = 1.f, a_rq = 0.f, b_rq = 0.f;
+  int relu2 = 0;
+  bool conv_input_is_converted = false;
+  int t_conv_in = -1;  // tensor or conversion buffer index actually read
+  // add
+  float add_a_rq = 0.f, add_b_rq = 0.f;
+  // dense
+  int dense_shape[5] = {1, 0, 0, 0, 0};
+  int perm[5] = {0, 1, 2, 3, 4};
+  bool has_perm = false;
+  // profiling
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  float last_ms = 0.f;
+};
+
+struct RbSlot {
+  Rulebook rb;
+  bool subm = false;
+  int coord_in = -1, coord_out = -1;
+  int ks[3], stride[3], pad[3], dil[3];
+  uint32_t max_out = 0;
+  bool initialised = false;
+};
+
+}  // namespace scn
+
+struct scn_engine {
+  std::vector<NodeDesc> nodes;
+  std::vector<TensorDesc> tdesc;
+  std::vector<int> inputs, outputs;
+  int precision = SCN_PRECISION_FP16;
+  unsigned flags = 0;
+  std::vector<RtTensor> tensors;      // graph tensors followed by conversion buffers
+  std::vector<CoordSet> coords;
+  std::vector<std::unique_ptr<RbSlot>> rulebooks;
+  std::vector<std::unique_ptr<ConvWeights>> convs;
+  std::vector<Step> steps;
+  std::map<std::string, int> tensor_by_name;
+  // input binding
+  const void* in_feat = nullptr;
+  const int32_t* in_idx = nullptr;
+  uint32_t in_n = 0, in_c = 0;
+  int in_grid[3] = {0, 0, 0};
+  const uint32_t* dds = nullptr;
+  DevBuf in_count;   // device uint32 holding N when no DDS pointer is bound
+  uint32_t input_cap = 0;
+  bool allocated = false;
+  int alloc_grid[3] = {0, 0, 0};
+  bool profiling = false;
+  bool input_set = false;
+  ~scn_engine() {
+    for (auto& s : steps) {
+      if (s.ev0) (void)hipEventDestroy(s.ev0);
+      if (s.ev1) (void)hipEventDestroy(s.ev1);
+    }
+  }
+};
+
+namespace scn {
+
+// ---------------------------------------------------------------------------------------------
+// planning
+// ---------------------------------------------------------------------------------------------
+struct Plan {
+  std::vector<int> comp, outp;             // per node effective precisions
+  std::vector<float> scale;                // per tensor, <= 0 when no consumer fixes one
+  std::vector<std::vector<std::pair<int, int>>> consumers;  // per tensor: (node, slot)
+};
+
+static Plan make_plan(const std::vector<NodeDesc>& nodes, size_t ntensors, int engine_precision) {
+  Plan p;
+  p.comp.assign(nodes.size(), SCN_PRECISION_FP16);
+  p.outp.assign(nodes.size(), SCN_PRECISION_FP16);
+  p.consumers.resize(ntensors);
+  for (size_t i = 0; i < nodes.size(); ++i) {
+    const NodeDesc& n = nodes[i];
+    for (size_t s = 0; s < n.in.size(); ++s) p.consumers[n.in[s]].push_back({(int)i, (int)s});
+    if (engine_precision != SCN_PRECISION_INT8) {
+      if ((n.op == Op::Conv || n.op == Op::Add) && n.precision == SCN_PRECISION_INT8)
+        SCN_LOGV("Ignore the layer[%s] precision[int8] because the model precision configured fp16", n.name.c_str());
+      continue;
+    }
+    if (n.op == Op::Conv) {
+      const bool ok = n.in_range > 0.f && (int)n.wranges.size() == n.wshape[0];
+      p.comp[i] = (n.precision == SCN_PRECISION_INT8 && ok) ? SCN_PRECISION_INT8 : SCN_PRECISION_FP16;
+      p.outp[i] = n.out_precision == SCN_PRECISION_INT8 ? SCN_PRECISION_INT8 : SCN_PRECISION_FP16;
+    } else if (n.op == Op::Add) {
+      const bool ok = n.a_range > 0.f && n.b_range > 0.f;
+      p.comp[i] = (n.precision == SCN_PRECISION_INT8 && ok) ? SCN_PRECISION_INT8 : SCN_PRECISION_FP16;
+      p.outp[i] = n.out_precision == SCN_PRECISION_INT8 ? SCN_PRECISION_INT8 : SCN_PRECISION_FP16;
+    }
+  }
+  // scale of a tensor = what its consumers expect: int8 conv first, then through Relu, then int8 Add,
+  // then an int8 ScatterDense range.
+  p.scale.assign(ntensors, -1.f);
+  std::vector<int> state(ntensors, 0);
+  std::function<float(int)> req = [&](int t) -> float {
+    if (state[t]) return p.scale[t];
+    state[t] = 1;
+    float res = -1.f;
+    for (auto& c : p.consumers[t]) {
+      const NodeDesc& n = nodes[c.first];
+      if (n.op == Op::Conv && p.comp[c.first] == SCN_PRECISION_INT8) {
+        res = n.in_range / 127.f;
+        break;
+      }
+    }
+    if (res <= 0.f)
+      for (auto& c : p.consumers[t]) {
+        const NodeDesc& n = nodes[c.first];
+        if (n.op == Op::Relu) {
+          res = req(n.out);
+          if (res > 0.f) break;
+        }
+      }
+    if (res <= 0.f)
+      for (auto& c : p.consumers[t]) {
+        const NodeDesc& n = nodes[c.first];
+        if (n.op == Op::Add && p.comp[c.first] == SCN_PRECISION_INT8) {
+          res = (c.second == 0 ? n.a_range : n.b_range) / 127.f;
+          break;
+        }
+      }
+    if (res <= 0.f)
+      for (auto& c : p.consumers[t]) {
+        const NodeDesc& n = nodes[c.first];
+        if (n.op == Op::Dense && n.dense_range > 0.f) {
+          res = n.dense_range / 127.f;
+          break;
+        }
+      }
+    p.scale[t] = res;
+    return res;
+  };
+  for (size_t t = 0; t < ntensors; ++t) req((int)t);
+  return p;
+}
+
+static uint32_t round_up(uint32_t v, uint32_t m) { return (v + m - 1) / m * m; }
+
+// ---------------------------------------------------------------------------------------------
+// build
+// ---------------------------------------------------------------------------------------------
+static bool build_engine(scn_engine& e) {
+  const auto& nodes = e.nodes;
+  const size_t nt = e.tdesc.size();
+  const bool keep_all = (e.flags & SCN_BUILD_KEEP_ALL) != 0;
+  Plan plan = make_plan(nodes, nt, e.precision);
+  e.tensors.reserve(nt + 2 * nodes.size() + 8);  // conversion buffers are appended; references stay valid
+  e.tensors.resize(nt);
+  std::set<int> graph_outputs(e.outputs.begin(), e.outputs.end());
+  if (e.inputs.size() != 1) {
+    set_error("the engine supports exactly one sparse input (got %zu)", e.inputs.size());
+    return false;
+  }
+  // ---- graph input
+  const int tin = e.inputs[0];
+  {
+    e.coords.emplace_back();
+    RtTensor& t = e.tensors[tin];
+    t.coord = 0;
+    t.dtype = SCN_DTYPE_FP16;
+    t.materialised = true;
+    // capacity of the input = output bound of its first convolution consumer
+    uint32_t cap = 0;
+    for (auto& c : plan.consumers[tin])
+      if (nodes[c.first].op == Op::Conv) cap = std::max(cap, nodes[c.first].max_out);
+    if (cap == 0) cap = 150000;
+    e.input_cap = cap;
+    e.coords[0].cap = cap;
+  }
+  Step s0;
+  s0.kind = StepKind::InputCount;
+  s0.label = "input";
+  e.steps.push_back(s0);
+
+  std::map<std::string, int> rb_by_key;
+  std::map<std::string, int> conversions;  // (tensor, dtype, scale, c) -> conversion buffer tensor
+  std::vector<bool> fused_away(nodes.size(), false);
+
+  auto ensure_table = [&](int coord, int node) {
+    // graph-input coordinates need an explicit hash build; strided outputs get theirs from the rulebook
+    CoordSet& cs = e.coords[coord];
+    if (cs.producer_rulebook >= 0) return;
+    for (auto& st : e.steps)
+      if (st.kind == StepKind::HashBuild && st.coord == coord) return;
+    Step st;
+    st.kind = StepKind::HashBuild;
+    st.coord = coord;
+    st.node = node;
+    st.label = "hash(input)";
+    e.steps.push_back(st);
+  };
+
+  auto single_consumer = [&](int t) -> int {
+    if (graph_outputs.count(t) || plan.consumers[t].size() != 1) return -1;
+    return plan.consumers[t][0].first;
+  };
+
+  for (size_t i = 0; i < nodes.size(); ++i) {
+    if (fused_away[i]) continue;
+    const NodeDesc& n = nodes[i];
+    switch (n.op) {
+      case Op::Conv: {
+        RtTensor& x = e.tensors[n.in[0]];
+        if (x.dense || x.coord < 0) {
+          set_error("node %s: input is not a sparse tensor", n.name.c_str());
+          return false;
+        }
+        const int cout = n.wshape[0], cin = n.wshape[4];
+        if (x.c == 0) x.c = cin;  // graph input: channel count comes from its first consumer
+        if (x.c != cin) {
+          set_error("node %s: input has %d channels, weight expects %d", n.name.c_str(), x.c, cin);
+          return false;
+        }
+        // rulebook
+        const std::string key = n.rulebook.empty() ? "" : std::string(n.subm ? "subm:" : "conv:") + n.rulebook;
+        int rbi = -1;
+        if (!key.empty() && rb_by_key.count(key)) {
+          rbi = rb_by_key[key];
+          RbSlot& slot = *e.rulebooks[rbi];
+          const bool same = slot.coord_in == x.coord && !memcmp(slot.ks, n.ks, 12) && !memcmp(slot.dil, n.dil, 12) &&
+                            (slot.subm || (!memcmp(slot.stride, n.stride, 12) && !memcmp(slot.pad, n.pad, 12)));
+          if (!same) {
+            SCN_LOGW("node %s: rulebook '%s' is shared with a different geometry or input; building a private one",
+                     n.name.c_str(), n.rulebook.c_str());
+            rbi = -1;
+          }
+        }
+        if (rbi < 0) {
+          ensure_table(x.coord, (int)i);
+          auto slot = std::make_unique<RbSlot>();
+          slot->subm = n.subm;
+          slot->coord_in = x.coord;
+          memcpy(slot->ks, n.ks, 12);
+          memcpy(slot->stride, n.stride, 12);
+          memcpy(slot->pad, n.pad, 12);
+          memcpy(slot->dil, n.dil, 12);
+          slot->max_out = n.max_out;
+          rbi = (int)e.rulebooks.size();
+          if (n.subm) {
+            slot->coord_out = x.coord;
+          } else {
+            e.coords.emplace_back();
+            CoordSet& oc = e.coords.back();
+            oc.cap = n.max_out;
+            oc.producer_rulebook = rbi;
+            slot->coord_out = (int)e.coords.size() - 1;
+          }
+          e.rulebooks.push_back(std::move(slot));
+          if (!key.empty() && !rb_by_key.count(key)) rb_by_key[key] = rbi;
+          Step st;
+          st.kind = n.subm ? StepKind::RulebookSubm : StepKind::RulebookSparse;
+          st.rulebook = rbi;
+          st.coord = x.coord;
+          st.coord_out = e.rulebooks[rbi]->coord_out;
+          st.node = (int)i;
+          st.label = std::string("rulebook(") + (n.rulebook.empty() ? n.name : n.rulebook) + ")";
+          e.steps.push_back(st);
+        }
+        RbSlot& slot = *e.rulebooks[rbi];
+        // weights
+        auto w = std::make_unique<ConvWeights>();
+        const int comp = plan.comp[i];
+        if (!w->init(n.weight.data(), n.wshape, comp == SCN_PRECISION_INT8 ? n.wranges.data() : nullptr,
+                     n.bias.empty() ? nullptr : n.bias.data(), comp))
+          return false;
+        const int ci = (int)e.convs.size();
+        // input form the kernel needs
+        Step st;
+        st.kind = StepKind::Conv;
+        st.node = (int)i;
+        st.label = n.name;
+        st.conv = ci;
+        st.rulebook = rbi;
+        st.coord = x.coord;
+        st.coord_out = slot.coord_out;
+        st.t_in = n.in[0];
+        const int want_dtype = comp == SCN_PRECISION_INT8 ? SCN_DTYPE_INT8 : SCN_DTYPE_FP16;
+        float want_scale = 1.f;
+        bool need_convert = false;
+        if (comp == SCN_PRECISION_INT8) {
+          if (x.dtype == SCN_DTYPE_INT8) {
+            st.x_scale = x.scale;
+          } else {
+            want_scale = n.in_range / 127.f;
+            st.x_scale = want_scale;
+            need_convert = true;
+          }
+        } else if (x.dtype == SCN_DTYPE_INT8) {
+          need_convert = true;  // dequantise
+        }
+        const bool is_graph_input = n.in[0] == tin;
+        if (!need_convert && (is_graph_input || x.ld < w->cin_pad)) need_convert = true;  // re-pad rows
+        st.t_conv_in = n.in[0];
+        if (need_convert) {
+          char keybuf[128];
+          snprintf(keybuf, sizeof(keybuf), "%d:%d:%a:%u", n.in[0], want_dtype, (double)want_scale, w->cin_pad);
+          auto it = conversions.find(keybuf);
+          if (it == conversions.end()) {
+            e.tensors.emplace_back();
+            RtTensor& cv = e.tensors.back();
+            RtTensor& xx = e.tensors[n.in[0]];  // (re-take: the vector may have grown)
+            cv.dtype = want_dtype;
+            cv.scale = want_scale;
+            cv.c = xx.c;
+            cv.ld = w->cin_pad;
+            cv.coord = xx.coord;
+            cv.materialised = true;
+            const int cvi = (int)e.tensors.size() - 1;
+            conversions[keybuf] = cvi;
+            Step cs;
+            cs.kind = StepKind::Convert;
+            cs.node = (int)i;
+            cs.label = std::string(want_dtype == SCN_DTYPE_INT8 ? "quantize(" : (xx.dtype == SCN_DTYPE_INT8 ? "dequantize(" : "pad(")) +
+                       e.tdesc[n.in[0]].name + ")";
+            cs.t_in = n.in[0];
+            cs.t_out = cvi;
+            cs.coord = xx.coord;
+            e.steps.push_back(cs);
+            st.t_conv_in = cvi;
+          } else {
+            st.t_conv_in = it->second;
+          }
+        }
+        // output tensor + fusion of a following Add (+Relu) / Relu
+        int t_out = n.out;
+        st.relu = n.activation == "ReLU" ? 1 : 0;
+        if (!n.activation.empty() && n.activation != "ReLU" && n.activation != "None")
+          SCN_LOGW("node %s: activation '%s' is not supported and is ignored", n.name.c_str(), n.activation.c_str());
+        int out_dtype = (plan.outp[i] == SCN_PRECISION_INT8 && plan.scale[n.out] > 0.f) ? SCN_DTYPE_INT8 : SCN_DTYPE_FP16;
+        float out_scale = out_dtype == SCN_DTYPE_INT8 ? plan.scale[n.out] : 1.f;
+        if (plan.outp[i] == SCN_PRECISION_INT8 && out_dtype != SCN_DTYPE_INT8)
+          SCN_LOGW("node %s: int8 output requested but no consumer provides a dynamic range; using fp16", n.name.c_str());
+        if (!keep_all) {
+          int c1 = single_consumer(n.out);
+          if (c1 >= 0 && nodes[c1].op == Op::Add && nodes[c1].in[0] != nodes[c1].in[1]) {
+            const NodeDesc& an = nodes[c1];
+            const int slot_a = an.in[0] == n.out ? 0 : 1;
+            const int other = an.in[1 - slot_a];
+            const RtTensor& ot = e.tensors[other];
+            // every node between the conv and the Add must be unrelated to the fusion and the
+            // residual must already exist
+            bool ok = ot.materialised && !ot.dense && ot.coord == slot.coord_out && ot.c == cout && c1 == (int)i + 1;
+            if (ok) {
+              st.fused_add = true;
+              st.t_in2 = other;
+              st.mid_dtype = out_dtype;
+              st.mid_scale = out_scale;
+              const bool add_i8 = plan.comp[c1] == SCN_PRECISION_INT8;
+              const float rq_self = add_i8 ? (slot_a == 0 ? an.a_range : an.b_range) / 127.f : 0.f;
+              const float rq_other = add_i8 ? (slot_a == 0 ? an.b_range : an.a_range) / 127.f : 0.f;
+              st.a_rq = (add_i8 && out_dtype == SCN_DTYPE_FP16) ? rq_self : 0.f;
+              st.b_rq = (add_i8 && ot.dtype == SCN_DTYPE_FP16) ? rq_other : 0.f;
+              fused_away[c1] = true;
+              e.tensors[n.out].coord = slot.coord_out;
+              e.tensors[n.out].c = cout;
+              t_out = an.out;
+              out_dtype = (plan.outp[c1] == SCN_PRECISION_INT8 && plan.scale[an.out] > 0.f) ? SCN_DTYPE_INT8 : SCN_DTYPE_FP16;
+              out_scale = out_dtype == SCN_DTYPE_INT8 ? plan.scale[an.out] : 1.f;
+              int c2 = single_consumer(an.out);
+              if (c2 >= 0 && nodes[c2].op == Op::Relu && c2 == c1 + 1) {
+                st.relu2 = 1;
+                fused_away[c2] = true;
+                e.tensors[an.out].coord = slot.coord_out;
+                e.tensors[an.out].c = cout;
+                t_out = nodes[c2].out;  // same dtype and scale as the Add output
+              }
+              st.label += "+" + an.name + (st.relu2 ? "+relu" : "");
+            }
+          } else if (c1 >= 0 && nodes[c1].op == Op::Relu && c1 == (int)i + 1 && !st.relu) {
+            st.relu = 1;
+            fused_away[c1] = true;
+            e.tensors[n.out].coord = slot.coord_out;
+            e.tensors[n.out].c = cout;
+            t_out = nodes[c1].out;
+            st.label += "+relu";
+          }
+        }
+        RtTensor& o = e.tensors[t_out];
+        o.dtype = out_dtype;
+        o.scale = out_scale;
+        o.c = cout;
+        o.ld = (uint32_t)w->mtiles * 16;
+        o.coord = slot.coord_out;
+        o.materialised = true;
+        st.t_out = t_out;
+        e.convs.push_back(std::move(w));
+        e.steps.push_back(st);
+        break;
+      }
+      case Op::Add: {
+        const RtTensor& a = e.tensors[n.in[0]];
+        const RtTensor& b = e.tensors[n.in[1]];
+        if (a.dense || b.dense || a.coord != b.coord || a.c != b.c || a.ld != b.ld) {
+          set_error("node %s: operands of Add must be sparse tensors on the same coordinates and channels", n.name.c_str());
+          return false;
+        }
+        Step st;
+        st.kind = StepKind::Add;
+        st.node = (int)i;
+        st.label = n.name;
+        st.t_in = n.in[0];
+        st.t_in2 = n.in[1];
+        st.coord = a.coord;
+        const bool add_i8 = plan.comp[i] == SCN_PRECISION_INT8;
+        st.add_a_rq = (add_i8 && a.dtype == SCN_DTYPE_FP16) ? n.a_range / 127.f : 0.f;
+        st.add_b_rq = (add_i8 && b.dtype == SCN_DTYPE_FP16) ? n.b_range / 127.f : 0.f;
+        int t_out = n.out;
+        const int out_dtype = (plan.outp[i] == SCN_PRECISION_INT8 && plan.scale[n.out] > 0.f) ? SCN_DTYPE_INT8 : SCN_DTYPE_FP16;
+        const float out_scale = out_dtype == SCN_DTYPE_INT8 ? plan.scale[n.out] : 1.f;
+        if (!keep_all) {
+          int c1 = single_consumer(n.out);
+          if (c1 >= 0 && nodes[c1].op == Op::Relu && c1 == (int)i + 1) {
+            st.relu = 1;
+            fused_away[c1] = true;
+            e.tensors[n.out].coord = a.coord;
+            e.tensors[n.out].c = a.c;
+            t_out = nodes[c1].out;
+            st.label += "+relu";
+          }
+        }
+        RtTensor& o = e.tensors[t_out];
+        o.dtype = out_dtype;
+        o.scale = out_scale;
+        o.c = a.c;
+        o.ld = a.ld;
+        o.coord = a.coord;
+        o.materialised = true;
+        st.t_out = t_out;
+        e.steps.push_back(st);
+        break;
+      }
+      case Op::Relu: {
+        const RtTensor& x = e.tensors[n.in[0]];
+        if (x.dense) {
+          set_error("node %s: Relu on a dense tensor is not supported", n.name.c_str());
+          return false;
+        }
+        Step st;
+        st.kind = StepKind::Relu;
+        st.node = (int)i;
+        st.label = n.name;
+        st.t_in = n.in[0];
+        st.t_out = n.out;
+        st.coord = x.coord;
+        RtTensor& o = e.tensors[n.out];
+        o.dtype = x.dtype;
+        o.scale = x.scale;
+        o.c = x.c;
+        o.ld = x.ld;
+        o.coord = x.coord;
+        o.materialised = true;
+        e.steps.push_back(st);
+        break;
+      }
+      case Op::Dense: {
+        const RtTensor& x = e.tensors[n.in[0]];
+        if (x.dense || n.out_shape.size() != 5 || n.out_shape[0] != 1 || n.out_shape[1] != x.c) {
+          set_error("node %s: ScatterDense needs a sparse input and output_shape [1, C=%d, D0, D1, D2]", n.name.c_str(), x.c);
+          return false;
+        }
+        Step st;
+        st.kind = StepKind::Dense;
+        st.node = (int)i;
+        st.label = n.name;
+        st.t_in = n.in[0];
+        st.coord = x.coord;
+        for (int j = 0; j < 5; ++j) st.dense_shape[j] = n.out_shape[j];
+        int t_out = n.out;
+        std::vector<int64_t> shape(n.out_shape.begin(), n.out_shape.end());
+        // fold a following Transpose (and Reshape views) into the scatter
+        if (!keep_all) {
+          int c1 = single_consumer(n.out);
+          if (c1 >= 0 && nodes[c1].op == Op::Transpose && nodes[c1].dims.size() == 5) {
+            bool okp = true;
+            bool seen[5] = {false, false, false, false, false};
+            for (int j = 0; j < 5; ++j) {
+              int64_t d = nodes[c1].dims[j];
+              if (d < 0 || d > 4 || seen[d]) okp = false; else seen[d] = true;
+            }
+            if (okp) {
+              st.has_perm = true;
+              std::vector<int64_t> ts(5);
+              for (int j = 0; j < 5; ++j) {
+                st.perm[j] = (int)nodes[c1].dims[j];
+                ts[j] = shape[st.perm[j]];
+              }
+              shape = ts;
+              fused_away[c1] = true;
+              e.tensors[n.out].dense = true;
+              t_out = nodes[c1].out;
+              st.label += "+" + nodes[c1].name;
+            }
+          }
+        }
+        RtTensor& o = e.tensors[t_out];
+        o.dense = true;
+        o.dtype = SCN_DTYPE_FP16;
+        o.shape = shape;
+        o.materialised = true;
+        st.t_out = t_out;
+        e.steps.push_back(st);
+        break;
+      }
+      case Op::Reshape: {
+        RtTensor& x = e.tensors[n.in[0]];
+        if (!x.dense) {
+          set_error("node %s: Reshape needs a dense input", n.name.c_str());
+          return false;
+        }
+        int64_t numel = 1, known = 1;
+        int infer = -1;
+        for (auto v : x.shape) numel *= v;
+        std::vector<int64_t> shape = n.dims;
+        for (size_t j = 0; j < shape.size(); ++j) {
+          if (shape[j] == -1) infer = (int)j; else known *= shape[j];
+        }
+        if (infer >= 0 && known > 0) shape[infer] = numel / known;
+        int64_t chk = 1;
+        for (auto v : shape) chk *= v;
+        if (chk != numel) {
+          set_error("node %s: Reshape to a different element count", n.name.c_str());
+          return false;
+        }
+        RtTensor& o = e.tensors[n.out];
+        o.dense = true;
+        o.dtype = x.dtype;
+        o.shape = shape;
+        o.view_of = x.view_of >= 0 ? x.view_of : n.in[0];
+        o.materialised = true;
+        break;
+      }
+      case Op::Transpose: {
+        set_error("node %s: a Transpose that does not directly follow ScatterDense is not supported", n.name.c_str());
+        return false;
+      }
+    }
+  }
+  for (size_t t = 0; t < nt; ++t) e.tensor_by_name[e.tdesc[t].name] = (int)t;
+  for (int o : e.outputs)
+    if (!e.tensors[o].materialised) {
+      set_error("output tensor %s is never produced", e.tdesc[o].name.c_str());
+      return false;
+    }
+  if (!e.in_count.alloc(64)) return false;
+  if (hipMemset(e.in_count.p, 0, 64) != hipSuccess) return false;
+  return true;
+}
+
+// Allocates everything whose size depends on the grid (first forward, or when the grid changes).
+static int allocate_runtime(scn_engine& e) {
+  CoordSet& c0 = e.coords[0];
+  memcpy(c0.grid, e.in_grid, 12);
+  if (!c0.own_table.buf.p && !c0.own_table.alloc_for(c0.cap)) return SCN_ERR_HIP;
+  // propagate grids and capacities through the strided rulebooks (they were created in order)
+  for (auto& up : e.rulebooks) {
+    RbSlot& s = *up;
+    const CoordSet& ci = e.coords[s.coord_in];
+    if (!s.subm) {
+      CoordSet& co = e.coords[s.coord_out];
+      uint64_t vol = 1;
+      for (int a = 0; a < 3; ++a) {
+        co.grid[a] = (ci.grid[a] + 2 * s.pad[a] - s.dil[a] * (s.ks[a] - 1) - 1) / s.stride[a] + 1;
+        SCN_REQUIRE(co.grid[a] >= 1, SCN_ERR_INVALID, "grid %dx%dx%d is too small for the network", e.in_grid[0],
+                    e.in_grid[1], e.in_grid[2]);
+        vol *= (uint64_t)co.grid[a];
+      }
+      co.cap = (uint32_t)std::min<uint64_t>(std::min<uint64_t>(s.max_out, vol), (uint64_t)ci.cap * 27ull);
+    }
+    const uint32_t max_in = ci.cap, max_out = s.subm ? ci.cap : e.coords[s.coord_out].cap;
+    const int kvol = s.ks[0] * s.ks[1] * s.ks[2];
+    if (!s.initialised || s.rb.max_in < max_in || s.rb.max_out < max_out) {
+      if (!s.rb.init(max_in, max_out, kvol)) return SCN_ERR_HIP;
+      s.initialised = true;
+    }
+  }
+  const bool keep_all = (e.flags & SCN_BUILD_KEEP_ALL) != 0;
+  for (size_t t = 0; t < e.tensors.size(); ++t) {
+    RtTensor& x = e.tensors[t];
+    if (!x.materialised || (int)t == e.inputs[0]) continue;
+    if (x.dense) {
+      if (x.view_of >= 0) continue;
+      size_t numel = 1;
+      for (auto v : x.shape) numel *= (size_t)v;
+      if (x.buf.bytes < numel * 2 && !x.buf.alloc(numel * 2)) return SCN_ERR_HIP;
+      x.data = x.buf.p;
+      continue;
+    }
+    const size_t rows = e.coords[x.coord].cap;
+    const size_t bytes = rows * x.ld * (x.dtype == SCN_DTYPE_INT8 ? 1 : 2);
+    if (x.buf.bytes < bytes) {
+      if (!x.buf.alloc(bytes)) return SCN_ERR_HIP;
+      SCN_HIP(hipMemset(x.buf.p, 0, bytes));
+    }
+    x.data = x.buf.p;
+  }
+  for (auto& x : e.tensors)
+    if (x.dense && x.view_of >= 0) x.data = e.tensors[x.view_of].data;
+  if (keep_all) {
+    for (auto& st : e.steps)
+      if (st.kind == StepKind::Conv) {
+        RtTensor& o = e.tensors[st.t_out];
+        const size_t bytes = (size_t)e.coords[o.coord].cap * o.ld * 4;
+        if (o.acc.bytes < bytes && !o.acc.alloc(bytes)) return SCN_ERR_HIP;
+      }
+  }
+  memcpy(e.alloc_grid, e.in_grid, 12);
+  e.allocated = true;
+  return SCN_OK;
+}
+
+static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
+  switch (st.kind) {
+    case StepKind::InputCount: {
+      CoordSet& c0 = e.coords[0];
+      uint32_t n = e.in_n;
+      if (n > c0.cap) {
+        SCN_LOGW("The number of input points %u exceeds the theoretical maximum number %u; truncate", n, c0.cap);
+        n = c0.cap;
+      }
+      c0.idx = e.in_idx;
+      c0.n_bound = n;
+      c0.table = nullptr;
+      int rc = set_count(e.in_count.as<uint32_t>(), e.dds, n, stream);
+      if (rc) return rc;
+      c0.n_dev = e.in_count.as<uint32_t>();
+      RtTensor& t = e.tensors[e.inputs[0]];
+      t.data = const_cast<void*>(e.in_feat);
+      t.ld = e.in_c;
+      return SCN_OK;
+    }
+    case StepKind::HashBuild: {
+      CoordSet& cs = e.coords[st.coord];
+      int rc = hash_build(cs.own_table, cs.idx, cs.n_bound, cs.n_dev, cs.grid, nullptr, stream);
+      if (rc) return rc;
+      cs.table = &cs.own_table;
+      return SCN_OK;
+    }
+    case StepKind::RulebookSubm: {
+      RbSlot& s = *e.rulebooks[st.rulebook];
+      CoordSet& cs = e.coords[s.coord_in];
+      return s.rb.build_subm(cs.idx, cs.n_bound, cs.n_dev, cs.grid, s.ks, s.dil, cs.table, stream);
+    }
+    case StepKind::RulebookSparse: {
+      RbSlot& s = *e.rulebooks[st.rulebook];
+      CoordSet& ci = e.coords[s.coord_in];
+      CoordSet& co = e.coords[s.coord_out];
+      int rc = s.rb.build_sparse(ci.idx, ci.n_bound, ci.n_dev, ci.grid, s.ks, s.stride, s.pad, s.dil, ci.table, stream);
+      if (rc) return rc;
+      co.idx = s.rb.out_indices;
+      co.n_dev = s.rb.n_out_dev();
+      co.n_bound = s.rb.n_bound_out;
+      co.table = &s.rb.out_table;
+      return SCN_OK;
+    }
+    case StepKind::Convert: {
+      const RtTensor& x = e.tensors[st.t_in];
+      RtTensor& o = e.tensors[st.t_out];
+      const CoordSet& cs = e.coords[x.coord];
+      return convert_rows(x.data, x.dtype, (uint32_t)x.c, x.ld, x.scale, o.data, o.dtype, o.ld, o.ld, o.scale, 0,
+                          cs.n_bound, cs.n_dev, stream);
+    }
+    case StepKind::Conv: {
+      const RtTensor& x = e.tensors[st.t_conv_in];
+      RtTensor& o = e.tensors[st.t_out];
+      RbSlot& s = *e.rulebooks[st.rulebook];
+      scn_conv_io io;
+      memset(&io, 0, sizeof(io));
+      io.x_dev = x.data;
+      io.x_ld = x.ld;
+      io.x_scale = st.x_scale;
+      io.relu = st.relu;
+      io.out_dtype = o.dtype;
+      io.out_scale = o.scale;
+      io.out_dev = o.data;
+      io.out_ld = o.ld;
+      io.acc_dev = o.acc.p;
+      if (st.fused_add) {
+        const RtTensor& r = e.tensors[st.t_in2];
+        io.res_dev = r.data;
+        io.res_dtype = r.dtype;
+        io.res_scale = r.scale;
+        io.res_ld = r.ld;
+        io.mid_dtype = st.mid_dtype;
+        io.mid_scale = st.mid_scale;
+        io.a_requant_scale = st.a_rq;
+        io.b_requant_scale = st.b_rq;
+        io.relu_after_add = st.relu2;
+      }
+      return conv_forward(*e.convs[st.conv], s.rb.nbr.as<int32_t>(), s.rb.ld, s.rb.n_out_dev(), s.rb.n_bound_out, io,
+                          stream);
+    }
+    case StepKind::Add: {
+      const RtTensor& a = e.tensors[st.t_in];
+      const RtTensor& b = e.tensors[st.t_in2];
+      RtTensor& o = e.tensors[st.t_out];
+      const CoordSet& cs = e.coords[a.coord];
+      return add_relu(a.data, a.dtype, a.scale, st.add_a_rq, b.data, b.dtype, b.scale, st.add_b_rq, o.data, o.dtype,
+                      o.scale, st.relu, a.ld, cs.n_bound, cs.n_dev, stream);
+    }
+    case StepKind::Relu: {
+      const RtTensor& x = e.tensors[st.t_in];
+      RtTensor& o = e.tensors[st.t_out];
+      const CoordSet& cs = e.coords[x.coord];
+      // value-preserving re-store with ReLU: int8 keeps its scale (q*s/s rounds back to q)
+      if (x.dtype == SCN_DTYPE_INT8)
+        return convert_rows(x.data, SCN_DTYPE_INT8, x.ld, x.ld, 1.f, o.data, SCN_DTYPE_INT8, o.ld, o.ld, 1.f, 1,
+                            cs.n_bound, cs.n_dev, stream);
+      return convert_rows(x.data, x.dtype, x.ld, x.ld, 1.f, o.data, o.dtype, o.ld, o.ld, 1.f, 1, cs.n_bound, cs.n_dev,
+                          stream);
+    }
+    case StepKind::Dense: {
+      const RtTensor& x = e.tensors[st.t_in];
+      RtTensor& o = e.tensors[st.t_out];
+      const CoordSet& cs = e.coords[x.coord];
+      return scatter_dense(x.data, x.dtype, x.scale, (uint32_t)x.c, x.ld, cs.idx, cs.n_bound, cs.n_dev, st.dense_shape,
+                           st.has_perm ? st.perm : nullptr, o.data, stream);
+    }
+  }
+  return SCN_ERR_INVALID;
+}
+
+// ---------------------------------------------------------------------------------------------
+// ONNX reading (protobuf wire format, only the messages the dialect uses)
+// field numbers: libraries/3DSparseConvolution/src/onnx/onnx-ml.proto:116-176,181-215,342-382,441-462,486-587
+// ---------------------------------------------------------------------------------------------
+struct PbReader {
+  const uint8_t* p;
+  const uint8_t* end;
+  bool ok = true;
+  PbReader(const uint8_t* b, size_t n) : p(b), end(b + n) {}
+  bool done() const { return p >= end || !ok; }
+  uint64_t varint() {
+    uint64_t v = 0;
+    int shift = 0;
+    while (p < end && shift < 64) {
+      const uint8_t b = *p++;
+      v |= (uint64_t)(b & 0x7f) << shift;
+      if (!(b & 0x80)) return v;
+      shift += 7;
+    }
+    ok = false;
+    return 0;
+  }
+  // reads one field header; for length-delimited fields sets [data, len)
+  bool next(int* field, int* wt, uint64_t* val, const uint8_t** data, size_t* len) {
+    if (done()) return false;
+    const uint64_t key = varint();
+    if (!ok) return false;
+    *field = (int)(key >> 3);
+    *wt = (int)(key & 7);
+    *val = 0;
+    *data = nullptr;
+    *len = 0;
+    switch (*wt) {
+      case 0: *val = varint(); break;
+      case 1:
+        if (end - p < 8) { ok = false; return false; }
+        memcpy(val, p, 8);
+        p += 8;
+        break;
+      case 2: {
+        const uint64_t n = varint();
+        if (!ok || (uint64_t)(end - p) < n) { ok = false; return false; }
+        *data = p;
+        *len = (size_t)n;
+        p += n;
+        break;
+      }
+      case 5: {
+        if (end - p < 4) { ok = false; return false; }
+        uint32_t v32;
+        memcpy(&v32, p, 4);
+        *val = v32;
+        p += 4;
+        break;
+      }
+      default: ok = false; return false;
+    }
+    return ok;
+  }
+};
+
+struct OnnxAttr {
+  std::string name, s;
+  float f = 0.f;
+  int64_t i = 0;
+  std::vector<float> floats;
+  std::vector<int64_t> ints;
+};
+struct OnnxNode {
+  std::string name, op_type;
+  std::vector<std::string> input, output;
+  std::vector<OnnxAttr> attrs;
+  const OnnxAttr* find(const char* n) const {
+    for (auto& a : attrs)
+      if (a.name == n) return &a;
+    return nullptr;
+  }
+};
+struct OnnxTensor {
+  std::string name;
+  std::vector<int64_t> dims;
+  int data_type = 0;
+  std::string raw;
+};
+struct OnnxGraph {
+  std::vector<OnnxNode> nodes;
+  std::vector<OnnxTensor> inits;
+  std::vector<std::string> inputs, outputs;
+};
+
+static bool parse_attr(const uint8_t* b, size_t n, OnnxAttr& a) {
+  PbReader r(b, n);
+  int f, wt;
+  uint64_t v;
+  const uint8_t* d;
+  size_t len;
+  while (r.next(&f, &wt, &v, &d, &len)) {
+    if (f == 1 && wt == 2) a.name.assign((const char*)d, len);
+    else if (f == 2 && wt == 5) { uint32_t u = (uint32_t)v; memcpy(&a.f, &u, 4); }
+    else if (f == 3 && wt == 0) a.i = (int64_t)v;
+    else if (f == 4 && wt == 2) a.s.assign((const char*)d, len);
+    else if (f == 7 && wt == 2) { for (size_t k = 0; k + 4 <= len; k += 4) { float x; memcpy(&x, d + k, 4); a.floats.push_back(x); } }
+    else if (f == 7 && wt == 5) { uint32_t u = (uint32_t)v; float x; memcpy(&x, &u, 4); a.floats.push_back(x); }
+    else if (f == 8 && wt == 2) { PbReader q(d, len); while (!q.done()) { uint64_t x = q.varint(); if (q.ok) a.ints.push_back((int64_t)x); } }
+    else if (f == 8 && wt == 0) a.ints.push_back((int64_t)v);
+  }
+  return r.ok;
+}
+
+static bool parse_node(const uint8_t* b, size_t n, OnnxNode& node) {
+  PbReader r(b, n);
+  int f, wt;
+  uint64_t v;
+  const uint8_t* d;
+  size_t len;
+  while (r.next(&f, &wt, &v, &d, &len)) {
+    if (wt != 2) continue;
+    if (f == 1) node.input.emplace_back((const char*)d, len);
+    else if (f == 2) node.output.emplace_back((const char*)d, len);
+    else if (f == 3) node.name.assign((const char*)d, len);
+    else if (f == 4) node.op_type.assign((const char*)d, len);
+    else if (f == 5) { OnnxAttr a; if (!parse_attr(d, len, a)) return false; node.attrs.push_back(std::move(a)); }
+  }
+  return r.ok;
+}
+
+static bool parse_tensor(const uint8_t* b, size_t n, OnnxTensor& t) {
+  PbReader r(b, n);
+  int f, wt;
+  uint64_t v;
+  const uint8_t* d;
+  size_t len;
+  while (r.next(&f, &wt, &v, &d, &len)) {
+    if (f == 1 && wt == 0) t.dims.push_back((int64_t)v);
+    else if (f == 1 && wt == 2) { PbReader q(d, len); while (!q.done()) { uint64_t x = q.varint(); if (q.ok) t.dims.push_back((int64_t)x); } }
+    else if (f == 2 && wt == 0) t.data_type = (int)v;
+    else if (f == 8 && wt == 2) t.name.assign((const char*)d, len);
+    else if (f == 9 && wt == 2) t.raw.assign((const char*)d, len);
+  }
+  return r.ok;
+}
+
+static bool parse_value_info_name(const uint8_t* b, size_t n, std::string& name) {
+  PbReader r(b, n);
+  int f, wt;
+  uint64_t v;
+  const uint8_t* d;
+  size_t len;
+  while (r.next(&f, &wt, &v, &d, &len))
+    if (f == 1 && wt == 2) name.assign((const char*)d, len);
+  return r.ok;
+}
+
+static bool parse_model(const std::string& bytes, OnnxGraph& g) {
+  PbReader r((const uint8_t*)bytes.data(), bytes.size());
+  int f, wt;
+  uint64_t v;
+  const uint8_t* d;
+  size_t len;
+  const uint8_t* gd = nullptr;
+  size_t glen = 0;
+  while (r.next(&f, &wt, &v, &d, &len))
+    if (f == 7 && wt == 2) { gd = d; glen = len; }
+  if (!r.ok || !gd) return false;
+  PbReader gr(gd, glen);
+  while (gr.next(&f, &wt, &v, &d, &len)) {
+    if (wt != 2) continue;
+    if (f == 1) { OnnxNode n; if (!parse_node(d, len, n)) return false; g.nodes.push_back(std::move(n)); }
+    else if (f == 5) { OnnxTensor t; if (!parse_tensor(d, len, t)) return false; g.inits.push_back(std::move(t)); }
+    else if (f == 11) { std::string s; if (!parse_value_info_name(d, len, s)) return false; g.inputs.push_back(s); }
+    else if (f == 12) { std::string s; if (!parse_value_info_name(d, len, s)) return false; g.outputs.push_back(s); }
+  }
+  return gr.ok;
+}
+
+}  // namespace scn
+
+// =============================================================================================
+// C ABI
+// =============================================================================================
+extern "C" {
+
+scn_builder* scn_builder_create(void) { return new scn_builder(); }
+void scn_builder_destroy(scn_builder* b) { delete b; }
+
+int scn_builder_push_input(scn_builder* b, const char* name) {
+  if (!b) return -1;
+  const int t = b->new_tensor(name, -1);
+  b->inputs.push_back(t);
+  return t;
+}
+
+static void copy3(int dst[3], const int* src, int dflt) {
+  for (int a = 0; a < 3; ++a) dst[a] = src ? src[a] : dflt;
+}
+
+int scn_builder_push_sparse_conv(scn_builder* b, const char* name, int x, const uint16_t* weight,
+                                 const int weight_shape[5], const float* weight_dynamic_ranges,
+                                 int n_weight_dynamic_ranges, const uint16_t* bias, int n_bias, const char* activation,
+                                 const int kernel_size[3], const int stride[3], const int padding[3],
+                                 const int dilation[3], float input_dynamic_range, int submanifold,
+                                 uint32_t max_output_points, uint32_t fixed_launch_points, const char* rulebook,
+                                 int precision, int output_precision, const char* output_name, int inverse) {
+  (void)fixed_launch_points;  // launch sizes always come from host-side bounds; nothing to fix
+  if (!b || !b->valid_tensor(x) || !weight || !weight_shape || !kernel_size) {
+    set_error("push_sparse_conv(%s): invalid arguments", name ? name : "");
+    return -1;
+  }
+  if (inverse) {
+    set_error("push_sparse_conv(%s): SparseInverseConvolution is not supported", name ? name : "");
+    return -1;
+  }
+  NodeDesc n;
+  n.op = Op::Conv;
+  n.name = name ? name : "";
+  n.in = {x};
+  size_t vol = 1;
+  for (int j = 0; j < 5; ++j) {
+    if (weight_shape[j] <= 0) {
+      set_error("push_sparse_conv(%s): invalid weight shape", n.name.c_str());
+      return -1;
+    }
+    n.wshape[j] = weight_shape[j];
+    vol *= (size_t)weight_shape[j];
+  }
+  if (weight_shape[1] != kernel_size[0] || weight_shape[2] != kernel_size[1] || weight_shape[3] != kernel_size[2]) {
+    set_error("push_sparse_conv(%s): weight shape [Cout,K0,K1,K2,Cin] does not match kernel_size", n.name.c_str());
+    return -1;
+  }
+  n.weight.assign(weight, weight + vol);
+  if (weight_dynamic_ranges && n_weight_dynamic_ranges > 0)
+    n.wranges.assign(weight_dynamic_ranges, weight_dynamic_ranges + n_weight_dynamic_ranges);
+  if (bias && n_bias > 0) {
+    if (n_bias != weight_shape[0]) {
+      set_error("push_sparse_conv(%s): bias has %d elements, Cout is %d", n.name.c_str(), n_bias, weight_shape[0]);
+      return -1;
+    }
+    n.bias.assign(bias, bias + n_bias);
+  }
+  n.activation = activation ? activation : "";
+  copy3(n.ks, kernel_size, 1);
+  copy3(n.stride, stride, 1);
+  copy3(n.pad, padding, 0);
+  copy3(n.dil, dilation, 1);
+  for (int a = 0; a < 3; ++a) {
+    if (n.stride[a] <= 0) n.stride[a] = 1;  // attributes missing from the model read as 0
+    if (n.dil[a] <= 0) n.dil[a] = 1;
+  }
+  n.in_range = input_dynamic_range;
+  n.subm = submanifold != 0;
+  n.max_out = max_output_points ? max_output_points : 150000;
+  n.rulebook = rulebook ? rulebook : "";
+  n.precision = precision;
+  n.out_precision = output_precision;
+  n.out = b->new_tensor(output_name, (int)b->nodes.size());
+  b->nodes.push_back(std::move(n));
+  return b->nodes.back().out;
+}
+
+int scn_builder_push_add(scn_builder* b, const char* name, int a, int b_tensor, float a_dynamic_range,
+                         float b_dynamic_range, const char* output_name, int precision, int output_precision,
+                         uint32_t fixed_launch_points) {
+  (void)fixed_launch_points;
+  if (!b || !b->valid_tensor(a) || !b->valid_tensor(b_tensor)) {
+    set_error("push_add(%s): invalid arguments", name ? name : "");
+    return -1;
+  }
+  NodeDesc n;
+  n.op = Op::Add;
+  n.name = name ? name : "";
+  n.in = {a, b_tensor};
+  n.a_range = a_dynamic_range;
+  n.b_range = b_dynamic_range;
+  n.precision = precision;
+  n.out_precision = output_precision;
+  n.out = b->new_tensor(output_name, (int)b->nodes.size());
+  b->nodes.push_back(std::move(n));
+  return b->nodes.back().out;
+}
+
+int scn_builder_push_relu(scn_builder* b, const char* name, int x, const char* output_name) {
+  if (!b || !b->valid_tensor(x)) {
+    set_error("push_relu(%s): invalid arguments", name ? name : "");
+    return -1;
+  }
+  NodeDesc n;
+  n.op = Op::Relu;
+  n.name = name ? name : "";
+  n.in = {x};
+  n.out = b->new_tensor(output_name, (int)b->nodes.size());
+  b->nodes.push_back(std::move(n));
+  return b->nodes.back().out;
+}
+
+int scn_builder_push_dense(scn_builder* b, const char* name, int x, const char* format, const char* output_name,
+                           const int input_spatial_shape[3], const int* output_shape, int n_output_shape,
+                           int output_layout, float input_dynamic_range, uint32_t input_bound) {
+  (void)input_bound;
+  if (!b || !b->valid_tensor(x) || !output_shape || n_output_shape <= 0) {
+    set_error("push_dense(%s): invalid arguments", name ? name : "");
+    return -1;
+  }
+  if (output_layout != 0 && output_layout != 1) {
+    set_error("push_dense(%s): only the NCHW output layout is supported (got %d)", name ? name : "", output_layout);
+    return -1;
+  }
+  NodeDesc n;
+  n.op = Op::Dense;
+  n.name = name ? name : "";
+  n.in = {x};
+  n.format = format ? format : "";
+  copy3(n.in_spatial, input_spatial_shape, 0);
+  n.out_shape.assign(output_shape, output_shape + n_output_shape);
+  n.dense_range = 0.f;  // int8 dense output is not supported: the dense tensor is always fp16
+  (void)input_dynamic_range;
+  n.out = b->new_tensor(output_name, (int)b->nodes.size());
+  b->nodes.push_back(std::move(n));
+  return b->nodes.back().out;
+}
+
+int scn_builder_push_reshape(scn_builder* b, const char* name, int x, const int64_t* shape, int n_shape,
+                             const char* output_name) {
+  if (!b || !b->valid_tensor(x) || !shape || n_shape <= 0) {
+    set_error("push_reshape(%s): invalid arguments", name ? name : "");
+    return -1;
+  }
+  NodeDesc n;
+  n.op = Op::Reshape;
+  n.name = name ? name : "";
+  n.in = {x};
+  n.dims.assign(shape, shape + n_shape);
+  n.out = b->new_tensor(output_name, (int)b->nodes.size());
+  b->nodes.push_back(std::move(n));
+  return b->nodes.back().out;
+}
+
+int scn_builder_push_transpose(scn_builder* b, const char* name, int x, const int64_t* dims, int n_dims,
+                               const char* output_name) {
+  if (!b || !b->valid_tensor(x) || !dims || n_dims <= 0) {
+    set_error("push_transpose(%s): invalid arguments", name ? name : "");
+    return -1;
+  }
+  NodeDesc n;
+  n.op = Op::Transpose;
+  n.name = name ? name : "";
+  n.in = {x};
+  n.dims.assign(dims, dims + n_dims);
+  n.out = b->new_tensor(output_name, (int)b->nodes.size());
+  b->nodes.push_back(std::move(n));
+  return b->nodes.back().out;
+}
+
+int scn_builder_push_output(scn_builder* b, int tensor) {
+  if (!b || !b->valid_tensor(tensor)) {
+    set_error("push_output: invalid tensor");
+    return SCN_ERR_INVALID;
+  }
+  b->outputs.push_back(tensor);
+  return SCN_OK;
+}
+
+scn_engine* scn_builder_build(scn_builder* b, int precision, unsigned flags, void* stream) {
+  (void)stream;
+  if (!b) return nullptr;
+  if (precision != SCN_PRECISION_FP16 && precision != SCN_PRECISION_INT8) {
+    set_error("build: precision must be Float16 (1) or Int8 (2)");
+    return nullptr;
+  }
+  auto* e = new scn_engine();
+  e->nodes = b->nodes;
+  e->tdesc = b->tensors;
+  e->inputs = b->inputs;
+  e->outputs = b->outputs;
+  e->precision = precision;
+  e->flags = flags;
+  if (!build_engine(*e)) {
+    delete e;
+    return nullptr;
+  }
+  SCN_LOGV("engine built: %zu nodes -> %zu steps, %zu rulebooks, precision %s", e->nodes.size(), e->steps.size(),
+           e->rulebooks.size(), precision == SCN_PRECISION_INT8 ? "int8" : "fp16");
+  return e;
+}
+
+static std::vector<int> attr_ints3(const OnnxNode& n, const char* name) {
+  std::vector<int> out;
+  if (const OnnxAttr* a = n.find(name))
+    for (auto v : a->ints) out.push_back((int)v);
+  return out;
+}
+
+scn_engine* scn_engine_create_from_onnx(const char* onnx_file, int precision, unsigned flags,
+                                        unsigned fixed_launch_points, void* stream) {
+  if (!onnx_file) return nullptr;
+  SCN_LOGV("Load onnx from: %s", onnx_file);
+  std::ifstream fin(onnx_file, std::ios::binary);
+  if (!fin) {
+    set_error("Parse onnx failed: %s (cannot open)", onnx_file);
+    return nullptr;
+  }
+  std::string bytes((std::istreambuf_iterator<char>(fin)), std::istreambuf_iterator<char>());
+  OnnxGraph g;
+  if (bytes.empty() || !parse_model(bytes, g)) {
+    set_error("Parse onnx failed: %s", onnx_file);
+    return nullptr;
+  }
+  std::unique_ptr<scn_builder, void (*)(scn_builder*)> b(scn_builder_create(), scn_builder_destroy);
+  std::map<std::string, int> tmap;
+  for (auto& name : g.inputs) {
+    bool is_init = false;
+    for (auto& t : g.inits) is_init |= t.name == name;
+    if (!is_init) tmap[name] = scn_builder_push_input(b.get(), name.c_str());
+  }
+  auto find_init = [&](const std::string& name, std::vector<uint16_t>& data, std::vector<int>& shape) -> bool {
+    for (auto& t : g.inits)
+      if (t.name == name) {
+        if (t.data_type != 10) {
+          set_error("Can not support non float data type[%d] for initializer data.", t.data_type);
+          return false;
+        }
+        size_t vol = 1;
+        shape.clear();
+        for (auto d : t.dims) { shape.push_back((int)d); vol *= (size_t)d; }
+        if (vol * 2 != t.raw.size()) {
+          set_error("Invalid parameter data size. %zu != %zu", vol * 2, t.raw.size());
+          return false;
+        }
+        data.resize(vol);
+        memcpy(data.data(), t.raw.data(), vol * 2);
+        return true;
+      }
+    set_error("Can not find initializer '%s' in ONNX.", name.c_str());
+    return false;
+  };
+  auto tensor_of = [&](const std::string& name) -> int {
+    auto it = tmap.find(name);
+    if (it == tmap.end()) {
+      set_error("tensor '%s' is used before it is produced", name.c_str());
+      return -1;
+    }
+    return it->second;
+  };
+  auto prec_of = [](const OnnxNode& n, const char* attr) {
+    const OnnxAttr* a = n.find(attr);
+    return (a && a->s == "int8") ? SCN_PRECISION_INT8 : SCN_PRECISION_FP16;
+  };
+  for (auto& n : g.nodes) {
+    unsigned flp = fixed_launch_points;
+    if (const OnnxAttr* a = n.find("fixed_launch_points")) flp = (unsigned)a->i;
+    int out = -1;
+    if (n.op_type == "SparseConvolution") {
+      if (n.input.size() < 3 || n.output.empty()) {
+        set_error("node %s: SparseConvolution needs inputs [x, weight, bias]", n.name.c_str());
+        return nullptr;
+      }
+      const int x = tensor_of(n.input[0]);
+      if (x < 0) return nullptr;
+      std::vector<uint16_t> w, bias;
+      std::vector<int> wshape, bshape;
+      if (!find_init(n.input[1], w, wshape) || !find_init(n.input[2], bias, bshape)) return nullptr;
+      if (wshape.size() != 5) {
+        set_error("node %s: weight must be [Cout,K0,K1,K2,Cin]", n.name.c_str());
+        return nullptr;
+      }
+      std::vector<float> wr;
+      if (const OnnxAttr* a = n.find("weight_dynamic_ranges")) wr = a->floats;
+      unsigned bound = 150000;
+      if (const OnnxAttr* a = n.find("output_bound")) bound = (unsigned)a->i;
+      else SCN_LOGV("using default output_bound: %u", bound);
+      const OnnxAttr* rb = n.find("rulebook");
+      const OnnxAttr* act = n.find("activation");
+      auto ks = attr_ints3(n, "kernel_size"), st = attr_ints3(n, "stride"), pd = attr_ints3(n, "padding"),
+           dl = attr_ints3(n, "dilation");
+      if (ks.size() != 3) {
+        set_error("node %s: kernel_size must have 3 entries", n.name.c_str());
+        return nullptr;
+      }
+      const OnnxAttr* idr = n.find("input_dynamic_range");
+      const OnnxAttr* subm = n.find("subm");
+      const OnnxAttr* inv = n.find("inverse");
+      out = scn_builder_push_sparse_conv(
+          b.get(), n.name.c_str(), x, w.data(), wshape.data(), wr.empty() ? nullptr : wr.data(), (int)wr.size(),
+          bias.data(), (int)bias.size(), act ? act->s.c_str() : "", ks.data(), st.size() == 3 ? st.data() : nullptr,
+          pd.size() == 3 ? pd.data() : nullptr, dl.size() == 3 ? dl.data() : nullptr, idr ? idr->f : 0.f,
+          subm ? (int)subm->i : 0, bound, flp, rb ? rb->s.c_str() : "", prec_of(n, "precision"),
+          prec_of(n, "output_precision"), n.output[0].c_str(), inv ? (int)inv->i : 0);
+    } else if (n.op_type == "Add" || n.op_type == "QuantAdd") {
+      if (n.input.size() < 2 || n.output.empty()) {
+        set_error("node %s: Add needs two inputs", n.name.c_str());
+        return nullptr;
+      }
+      const int a = tensor_of(n.input[0]), c = tensor_of(n.input[1]);
+      if (a < 0 || c < 0) return nullptr;
+      const OnnxAttr* r0 = n.find("input0_dynamic_range");
+      const OnnxAttr* r1 = n.find("input1_dynamic_range");
+      out = scn_builder_push_add(b.get(), n.name.c_str(), a, c, r0 ? r0->f : 0.f, r1 ? r1->f : 0.f, n.output[0].c_str(),
+                                 prec_of(n, "precision"), prec_of(n, "output_precision"), fixed_launch_points);
+    } else if (n.op_type == "Relu") {
+      const int x = n.input.empty() ? -1 : tensor_of(n.input[0]);
+      if (x < 0 || n.output.empty()) return nullptr;
+      out = scn_builder_push_relu(b.get(), n.name.c_str(), x, n.output[0].c_str());
+    } else if (n.op_type == "ScatterDense") {
+      const int x = n.input.empty() ? -1 : tensor_of(n.input[0]);
+      if (x < 0 || n.output.empty()) return nullptr;
+      auto iss = attr_ints3(n, "input_spatial_shape");
+      auto os = attr_ints3(n, "output_shape");
+      const OnnxAttr* fmt = n.find("format");
+      const OnnxAttr* idr = n.find("input_dynamic_range");
+      const OnnxAttr* lay = n.find("output_layout");
+      int layout = 1;
+      if (lay && lay->s == "NCHW32") layout = 2;
+      else if (lay && lay->s == "NHWzC") layout = 3;
+      out = scn_builder_push_dense(b.get(), n.name.c_str(), x, fmt ? fmt->s.c_str() : "", n.output[0].c_str(),
+                                   iss.size() == 3 ? iss.data() : nullptr, os.data(), (int)os.size(), layout,
+                                   idr ? idr->f : 0.f, fixed_launch_points);
+    } else if (n.op_type == "Reshape" || n.op_type == "Transpose") {
+      const int x = n.input.empty() ? -1 : tensor_of(n.input[0]);
+      if (x < 0 || n.output.empty()) return nullptr;
+      std::vector<int64_t> dims;
+      if (const OnnxAttr* a = n.find("dims")) dims = a->ints;
+      out = n.op_type == "Reshape"
+                ? scn_builder_push_reshape(b.get(), n.name.c_str(), x, dims.data(), (int)dims.size(), n.output[0].c_str())
+                : scn_builder_push_transpose(b.get(), n.name.c_str(), x, dims.data(), (int)dims.size(), n.output[0].c_str());
+    } else {
+      set_error("Unsupport operator [%s]", n.op_type.c_str());
+      return nullptr;
+    }
+    if (out < 0) return nullptr;
+    tmap[n.output[0]] = out;
+  }
+  for (auto& name : g.outputs) {
+    const int t = tensor_of(name);
+    if (t < 0) return nullptr;
+    scn_builder_push_output(b.get(), t);
+  }
+  return scn_builder_build(b.get(), precision, flags, stream);
+}
+
+void scn_engine_destroy(scn_engine* e) { delete e; }
+int scn_engine_num_input(const scn_engine* e) { return e ? (int)e->inputs.size() : 0; }
+int scn_engine_num_output(const scn_engine* e) { return e ? (int)e->outputs.size() : 0; }
+
+int scn_engine_set_input(scn_engine* e, int index, const void* features_fp16_dev, uint32_t n, uint32_t channels,
+                         const int32_t* indices_dev, const int grid_size[3]) {
+  SCN_REQUIRE(e && index == 0 && grid_size, SCN_ERR_INVALID, "set_input: invalid engine / index");
+  SCN_REQUIRE((features_fp16_dev && indices_dev) || n == 0, SCN_ERR_INVALID, "set_input: null pointers with n > 0");
+  const RtTensor& t = e->tensors[e->inputs[0]];
+  SCN_REQUIRE(t.c == 0 || (uint32_t)t.c == channels, SCN_ERR_INVALID, "set_input: the model expects %d input channels, got %u",
+              t.c, channels);
+  SCN_REQUIRE(((uintptr_t)indices_dev & 15) == 0, SCN_ERR_INVALID, "set_input: indices must be 16-byte aligned");
+  e->in_feat = features_fp16_dev;
+  e->in_idx = indices_dev;
+  e->in_n = n;
+  e->in_c = channels;
+  memcpy(e->in_grid, grid_size, 12);
+  e->input_set = true;
+  return SCN_OK;
+}
+
+int scn_engine_set_num_points_device_ptr(scn_engine* e, int index, const uint32_t* n_dev) {
+  SCN_REQUIRE(e && index == 0, SCN_ERR_INVALID, "set_num_points_device_ptr: invalid engine / index");
+  e->dds = n_dev;
+  return SCN_OK;
+}
+
+int scn_engine_forward(scn_engine* e, void* stream_) {
+  SCN_REQUIRE(e, SCN_ERR_INVALID, "forward: null engine");
+  SCN_REQUIRE(e->input_set, SCN_ERR_INVALID, "forward: no input has been set");
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!e->allocated || memcmp(e->alloc_grid, e->in_grid, 12) != 0) {
+    int rc = allocate_runtime(*e);
+    if (rc) return rc;
+  }
+  for (auto& st : e->steps) {
+    if (e->profiling) {
+      if (!st.ev0) {
+        SCN_HIP(hipEventCreate(&st.ev0));
+        SCN_HIP(hipEventCreate(&st.ev1));
+      }
+      SCN_HIP(hipEventRecord(st.ev0, stream));
+    }
+    int rc = run_step(*e, st, stream);
+    if (rc) {
+      SCN_LOGE("forward failed at step %s", st.label.c_str());
+      return rc;
+    }
+    if (e->profiling) SCN_HIP(hipEventRecord(st.ev1, stream));
+  }
+  if (e->profiling) {
+    SCN_HIP(hipStreamSynchronize(stream));
+    for (auto& st : e->steps) SCN_HIP(hipEventElapsedTime(&st.last_ms, st.ev0, st.ev1));
+  }
+  return SCN_OK;
+}
+
+static void fill_view(scn_engine* e, int t, scn_tensor_view* v) {
+  const RtTensor& x = e->tensors[t];
+  memset(v, 0, sizeof(*v));
+  v->name = (t < (int)e->tdesc.size()) ? e->tdesc[t].name.c_str() : "";
+  v->features_dev = x.data;
+  v->dtype = x.dtype;
+  v->scale = x.scale;
+  if (x.dense) {
+    v->ndim = (int)std::min<size_t>(x.shape.size(), 8);
+    for (int j = 0; j < v->ndim; ++j) v->shape[j] = x.shape[j];
+  } else {
+    const CoordSet& cs = e->coords[x.coord];
+    v->ndim = 2;
+    v->shape[0] = cs.n_bound;
+    v->shape[1] = x.ld;
+    v->indices_dev = cs.idx;
+    v->num_dev = cs.n_dev;
+    memcpy(v->grid_size, cs.grid, 12);
+  }
+}
+
+int scn_engine_output(scn_engine* e, int index, scn_tensor_view* view) {
+  SCN_REQUIRE(e && view && index >= 0 && index < (int)e->outputs.size(), SCN_ERR_INVALID, "output: invalid index");
+  fill_view(e, e->outputs[index], view);
+  return SCN_OK;
+}
+
+int scn_engine_tensor(scn_engine* e, const char* name, scn_tensor_view* view, void** acc_dev) {
+  SCN_REQUIRE(e && name && view, SCN_ERR_INVALID, "tensor: invalid arguments");
+  auto it = e->tensor_by_name.find(name);
+  SCN_REQUIRE(it != e->tensor_by_name.end(), SCN_ERR_INVALID, "tensor '%s' does not exist", name);
+  SCN_REQUIRE(e->tensors[it->second].materialised, SCN_ERR_INVALID,
+              "tensor '%s' was fused away (build with SCN_BUILD_KEEP_ALL to keep it)", name);
+  fill_view(e, it->second, view);
+  if (acc_dev) *acc_dev = e->tensors[it->second].acc.p;
+  return SCN_OK;
+}
+
+int scn_engine_set_profiling(scn_engine* e, int enabled) {
+  SCN_REQUIRE(e, SCN_ERR_INVALID, "null engine");
+  e->profiling = enabled != 0;
+  return SCN_OK;
+}
+int scn_engine_num_nodes(const scn_engine* e) { return e ? (int)e->steps.size() : 0; }
+int scn_engine_node_info(scn_engine* e, int node, const char** name, const char** kind, float* last_ms) {
+  SCN_REQUIRE(e && node >= 0 && node < (int)e->steps.size(), SCN_ERR_INVALID, "node_info: invalid index");
+  static const char* kinds[] = {"input", "hash", "rulebook_subm", "rulebook_sparse", "convert", "conv", "add", "relu", "dense"};
+  const Step& s = e->steps[node];
+  if (name) *name = s.label.c_str();
+  if (kind) *kind = kinds[(int)s.kind];
+  if (last_ms) *last_ms = s.last_ms;
+  return SCN_OK;
+}
+
+}  // extern "C"

@@ -375,6 +375,12 @@ __global__ void k_set_count(uint32_t* dst, const uint32_t* n_dev, uint32_t n_bou
   }
 }
 
+int set_count(uint32_t* dst, const uint32_t* n_dev, uint32_t n_bound, hipStream_t stream) {
+  hipLaunchKernelGGL(k_set_count, dim3(1), dim3(64), 0, stream, dst, n_dev, n_bound);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
 static int launch_build_nbr(const Rulebook& rb, const int32_t* out_coords, uint32_t n_bound, bool identity_center,
                             hipStream_t stream) {
   if (n_bound == 0) return SCN_OK;

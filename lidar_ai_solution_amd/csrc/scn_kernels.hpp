@@ -76,6 +76,7 @@ struct ConvWeights {
 int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, const uint32_t* n_out_dev,
                  uint32_t n_bound, const scn_conv_io& io, hipStream_t stream);
 
+int set_count(uint32_t* dst, const uint32_t* n_dev, uint32_t n_bound, hipStream_t stream);
 int fill_u32(void* p, uint32_t value, size_t count, hipStream_t stream);
 int hash_build(const CoordTable& t, const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3],
                uint32_t* n_eff_out, hipStream_t stream);

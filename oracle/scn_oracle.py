@@ -317,11 +317,15 @@ def tensor_scales(graph, prec):
 
 
 def run_graph(graph, features_f16: np.ndarray, indices: np.ndarray, grid, precision: str = "fp16",
-              record: Optional[dict] = None):
+              record: Optional[dict] = None, override: Optional[dict] = None):
     """Walks the graph.  Returns {output name: ndarray (dense) or SparseT}.
 
     record, when given, receives per node name a dict with the rulebook, the accumulators (`acc`)
     and the stored output (`out`, plus `scale` for int8) of that node.
+    override maps a tensor name to stored features that replace what the walk computed for that
+    tensor (same dtype and shape).  Tests use it to re-base the walk on the device's own output of
+    an fp16-computed node, whose summation order the oracle does not model, so that every int8 node
+    downstream sees identical inputs and can be compared bit for bit.
     """
     prec = node_precisions(graph, precision)
     scales = tensor_scales(graph, prec)
@@ -420,6 +424,13 @@ def run_graph(graph, features_f16: np.ndarray, indices: np.ndarray, grid, precis
                 rec.update(out=T[n.outputs[0]])
         else:
             raise ValueError(f"Unsupport operator [{n.op_type}]")
+        if override and n.outputs[0] in override and isinstance(T[n.outputs[0]], SparseT):
+            t = T[n.outputs[0]]
+            new = np.ascontiguousarray(override[n.outputs[0]])[:, :t.feat.shape[1]]
+            assert new.dtype == t.feat.dtype and new.shape == t.feat.shape, n.name
+            t.feat = new
+            if rec is not None:
+                rec["out"] = new
         if record is not None:
             record[n.name] = rec
     return {name: T[name] for name in graph.outputs}
