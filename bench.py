@@ -1,0 +1,328 @@
+#!/usr/bin/env python3
+"""Benchmark of the SCN lidar backbone on one MI355X.
+
+A step is one Engine.forward of the int8 CenterPoint-shaped backbone over one synthetic lidar frame
+(~120 k active voxels, already voxelized and resident in HBM), the configuration the headline metric
+is quoted on.  Prints ONE JSON line: frames/s (value), active voxels/s, per-step times, the roofline
+position of the dominant kernel (durations measured here with HIP events on the launch stream) and
+the CPU oracle timed on the same frame on this machine's host cores.
+
+    python bench.py --gpus 1 --steps 200 --warmup 20
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+INT8_PEAK_TOPS = 5000.0        # dense int8 MFMA, published
+FP16_PEAK_TFLOPS = 2500.0
+GRID_ZYX = (41, 1440, 1440)
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--precision", default="int8", choices=["int8", "fp16"])
+    ap.add_argument("--points", type=int, default=250000)
+    ap.add_argument("--no-graph", action="store_true", help="launch kernels directly instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-reps", type=int, default=3)
+    ap.add_argument("--layers", action="store_true", help="also print the per-step table to stderr")
+    return ap.parse_args()
+
+
+def voxelize_on_gpu(points_np, order="zyx"):
+    import torch
+    from lidar_ai_solution_amd import synth
+    from lidar_ai_solution_amd.scn import Voxelization
+    vox = Voxelization(synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, max_voxels=synth.MAX_VOXELS,
+                       max_points=max(synth.MAX_POINTS, points_np.shape[0]))
+    pts = torch.from_numpy(points_np.view(np.int16)).cuda().view(torch.float16)
+    vox.forward(pts, order=order)
+    nv = vox.num_voxels()
+    feats = torch.empty((nv, 5), dtype=torch.float16, device="cuda")
+    idx = torch.empty((nv, 4), dtype=torch.int32, device="cuda")
+    hip = __import__("lidar_ai_solution_amd.capi", fromlist=["x"]).hip_runtime()
+    hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+    torch.cuda.synchronize()
+    assert hip.hipMemcpy(C.c_void_p(feats.data_ptr()), C.c_void_p(vox.features_ptr()), nv * 10, 3) == 0
+    assert hip.hipMemcpy(C.c_void_p(idx.data_ptr()), C.c_void_p(vox.indices_ptr()), nv * 16, 3) == 0
+    # voxelization time (its own small loop, reported separately from the backbone)
+    for _ in range(5):
+        vox.forward(pts, order=order)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    reps = 50
+    for _ in range(reps):
+        vox.forward(pts, order=order)
+    torch.cuda.synchronize()
+    vox_ms = (time.perf_counter() - t0) / reps * 1e3
+    return feats, idx, nv, vox_ms, vox
+
+
+def stage_pair_counts(eng_keep, graph):
+    """Rulebook pair count per conv node, recomputed with the stage-level C ABI on the coordinates of
+    each conv's input tensor (the engine does not expose its neighbour tables)."""
+    import torch
+    from lidar_ai_solution_amd import capi
+    L = capi.lib()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    cache = {}
+    out = {}
+    for n in graph.nodes:
+        if n.op_type != "SparseConvolution":
+            continue
+        a = n.attrs
+        key = (n.inputs[0] if not a.get("rulebook") else ("subm" if a.get("subm") else "conv") + a["rulebook"],
+               tuple(a["kernel_size"]), tuple(a["stride"]), tuple(a["padding"]), int(a.get("subm", 0)))
+        if key not in cache:
+            view, _ = eng_keep.tensor(n.inputs[0]) if n.inputs[0] != graph.inputs[0] else (None, None)
+            if view is None:
+                idx_ptr, n_rows, grid = eng_keep._keep[1].data_ptr(), int(eng_keep._keep[1].shape[0]), GRID_ZYX
+            else:
+                idx_ptr, n_rows, grid = view.indices_ptr, view.num_rows(), view.grid_size
+            kvol = int(np.prod(a["kernel_size"]))
+            rb = L.scn_rulebook_create(max(n_rows, 1), max(n_rows, int(a.get("output_bound", 200000))), kvol)
+            g3 = capi.i3(*grid)
+            if a.get("subm"):
+                capi.check(L.scn_rulebook_build_subm(rb, C.c_void_p(idx_ptr), n_rows, None, g3, capi.i3(*a["kernel_size"]),
+                                                     capi.i3(*a["dilation"]), st))
+            else:
+                capi.check(L.scn_rulebook_build_sparse(rb, C.c_void_p(idx_ptr), n_rows, None, g3, capi.i3(*a["kernel_size"]),
+                                                       capi.i3(*a["stride"]), capi.i3(*a["padding"]), capi.i3(*a["dilation"]), st))
+            offs = torch.zeros(kvol + 1, dtype=torch.int64, device="cuda")
+            scratch = torch.empty(1, dtype=torch.int32, device="cuda")
+            capi.check(L.scn_rulebook_pairs(rb, C.c_void_p(scratch.data_ptr()), C.c_void_p(scratch.data_ptr()),
+                                            C.c_void_p(offs.data_ptr()), 0, st))
+            torch.cuda.synchronize()
+            o = offs.cpu().numpy()
+            n_out_t = torch.empty(1, dtype=torch.int32, device="cuda")
+            hip = capi.hip_runtime()
+            hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+            hip.hipMemcpy(C.c_void_p(n_out_t.data_ptr()), C.c_void_p(L.scn_rulebook_num_out_dev(rb)), 4, 3)
+            cache[key] = (int(o[-1]), n_rows, int(n_out_t.cpu().numpy()[0]), int((np.diff(o) == 0).sum()))
+            L.scn_rulebook_destroy(rb)
+        out[n.name] = cache[key]
+    return out
+
+
+def conv_algorithmic(node, graph, pairs, n_in, n_out, e_in, e_out, e_w, residual_bytes=0):
+    """Algorithmic bytes and ops of one convolution launch: every input row read once, every output
+    row written once, 8 bytes per rulebook pair, weights once, bias + scale once."""
+    w = graph.initializers[node.inputs[1]]
+    cout, cin = w.shape[0], w.shape[-1]
+    kvol = int(np.prod(w.shape[1:4]))
+    nbytes = n_in * cin * e_in + n_out * cout * e_out + pairs * 8 + kvol * cin * cout * e_w + cout * 6 + residual_bytes
+    ops = 2 * pairs * cin * cout
+    return nbytes, ops
+
+
+def node_io_bytes(node, graph, precision, fused_add, n_out):
+    """Element sizes (input, output, weight) of one convolution under the engine's precision rules and
+    the bytes of the residual operand when the following Add is fused into it."""
+    cout = graph.initializers[node.inputs[1]].shape[0]
+    if precision != "int8":
+        return 2, 2, 2, (n_out * cout * 2 if fused_add else 0)
+    comp_i8 = node.attrs.get("precision", "") == "int8"
+    out_i8 = node.attrs.get("output_precision", "") == "int8"
+    e = 1 if comp_i8 else 2
+    e_out = 1 if out_i8 else 2
+    return e, e_out, e, (n_out * cout * e_out if fused_add else 0)
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every box of this build has a single MI355X and frames are independent, "
+              "so N GPUs would run N independent engines; run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from lidar_ai_solution_amd import capi, graphs, synth
+    from lidar_ai_solution_amd.calibrate import calibrate_amax, gpu_runner
+    from lidar_ai_solution_amd.scn import Engine
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    capi.lib().scn_set_log_level(2)
+    torch.cuda.set_device(0)
+    t_setup = time.perf_counter()
+
+    # ---- workload: BASELINE.json configs[2] (int8 CenterPoint-shaped backbone, ~120k voxels)
+    frame = synth.lidar_frame(seed=0, n_points=args.points)
+    feats, idx, nvox, vox_ms, vox = voxelize_on_gpu(frame, "zyx")
+    graph, tags = graphs.centerpoint_scn(seed=0)
+    if args.precision == "int8":
+        calib = []
+        for s in range(1, 5):  # 4 seeded calibration frames
+            f_c, i_c, _, _, v_c = voxelize_on_gpu(synth.lidar_frame(seed=100 + s, n_points=args.points), "zyx")
+            calib.append((f_c.cpu().numpy(), i_c.cpu().numpy()))
+            v_c.close()
+        amax = calibrate_amax(graph, calib, GRID_ZYX, gpu_runner)
+        graphs.apply_int8_plan(graph, tags, amax, "centerpoint")
+    eng = Engine.from_graph(graph, args.precision)
+    eng.set_input(feats, idx, GRID_ZYX)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        eng.forward()            # first call allocates; later calls only launch
+        eng.forward()
+    torch.cuda.synchronize()
+
+    # ---- per-step times (HIP events on the launch stream), averaged over a few profiled forwards
+    eng.set_profiling(True)
+    prof_reps = 20
+    acc_ms = None
+    with torch.cuda.stream(stream):
+        for _ in range(prof_reps):
+            eng.forward()
+            t = eng.step_times()
+            acc_ms = [x[2] for x in t] if acc_ms is None else [a + x[2] for a, x in zip(acc_ms, t)]
+    steps_info = [(t[i][0], t[i][1], acc_ms[i] / prof_reps) for i in range(len(t))]
+    eng.set_profiling(False)
+
+    # ---- timed region
+    use_graph = not args.no_graph
+    graph_obj = None
+    if use_graph:
+        graph_obj = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            eng.forward()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph_obj, stream=stream):
+            eng.forward()
+        torch.cuda.synchronize()
+
+    def step():
+        if graph_obj is not None:
+            graph_obj.replay()
+        else:
+            eng.forward()
+
+    with torch.cuda.stream(stream):
+        for _ in range(args.warmup):
+            step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    with torch.cuda.stream(stream):
+        for _ in range(args.steps):
+            step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    out_view = eng.output(0)
+    checksum = float(out_view.torch().float().abs().sum().item())
+
+    # ---- roofline of the dominant kernel
+    keep = Engine.from_graph(graph, args.precision, keep_all=True)
+    keep.set_input(feats, idx, GRID_ZYX)
+    keep.forward()
+    torch.cuda.synchronize()
+    pair_info = stage_pair_counts(keep, graph)
+    keep.close()
+    conv_nodes = {n.name: n for n in graph.nodes if n.op_type == "SparseConvolution"}
+    groups = {}
+    total_ops = 0
+    total_bytes = 0
+    layer_rows = []
+    for label, kind, ms in steps_info:
+        if kind != "conv":
+            continue
+        name = label.split("+")[0]
+        node = conv_nodes[name]
+        pairs, n_in, n_out, empty = pair_info[name]
+        e_in, e_out, e_w, res = node_io_bytes(node, graph, args.precision, fused_add="+add" in label, n_out=n_out)
+        nbytes, ops = conv_algorithmic(node, graph, pairs, n_in, n_out, e_in, e_out, e_w, res)
+        w = graph.initializers[node.inputs[1]]
+        key = (w.shape[-1], w.shape[0], int(node.attrs.get("subm", 0)), tuple(node.attrs["kernel_size"]))
+        g = groups.setdefault(key, {"ms": 0.0, "bytes": 0, "ops": 0, "launches": 0})
+        g["ms"] += ms
+        g["bytes"] += nbytes
+        g["ops"] += ops
+        g["launches"] += 1
+        total_ops += ops
+        total_bytes += nbytes
+        layer_rows.append((label, ms * 1e3, pairs, n_out, nbytes, ops))
+    dom_key, dom = max(groups.items(), key=lambda kv: kv[1]["ms"])
+    dom_ms = dom["ms"] / dom["launches"]
+    dom_bytes = dom["bytes"] / dom["launches"]
+    dom_ops = dom["ops"] / dom["launches"]
+    achieved_gbs = dom_bytes / (dom_ms * 1e-3) / 1e9
+    achieved_tops = dom_ops / (dom_ms * 1e-3) / 1e12
+    roofline = {
+        "bound": "hbm", "achieved": round(achieved_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(achieved_gbs / HBM_PEAK_GBS, 5), "traffic": None,
+        "kernel": f"k_conv_rows {args.precision} Cin={dom_key[0]} Cout={dom_key[1]} {'subm' if dom_key[2] else 'strided'} k={'x'.join(map(str, dom_key[3]))}",
+        "launches_per_frame": dom["launches"], "avg_launch_us": round(dom_ms * 1e3, 2),
+        "algorithmic_bytes_per_launch": int(dom_bytes), "ops_per_launch": int(dom_ops),
+        "mfma_achieved_TOPs": round(achieved_tops, 3),
+        "mfma_frac_of_peak": round(achieved_tops / (INT8_PEAK_TOPS if args.precision == "int8" else FP16_PEAK_TFLOPS), 6),
+    }
+    sum_step_ms = sum(x[2] for x in steps_info)
+    by_kind = {}
+    for label, kind, ms in steps_info:
+        by_kind[kind] = by_kind.get(kind, 0.0) + ms
+
+    # ---- CPU baseline: the scalar/OpenMP oracle on the same frame, on this machine's host cores
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import scn_oracle as O
+        f_np, i_np = feats.cpu().numpy(), idx.cpu().numpy()
+        O.run_graph(graph, f_np, i_np, GRID_ZYX, args.precision)  # warm-up
+        ts = []
+        for _ in range(args.cpu_reps):
+            c0 = time.perf_counter()
+            O.run_graph(graph, f_np, i_np, GRID_ZYX, args.precision)
+            ts.append(time.perf_counter() - c0)
+        med = float(np.median(ts))
+        cpu = {"value": round(1.0 / med, 4), "unit": "frames/s", "cores": O.num_threads(), "kind": "port",
+               "sample": f"same {nvox}-voxel frame, median of {args.cpu_reps} full backbone passes after 1 warm-up "
+                         f"(rulebooks + int8 GEMM + epilogue, OpenMP over rulebook pairs)",
+               "ms_per_frame": round(med * 1e3, 1), "voxels_per_s": round(nvox / med, 1)}
+
+    if args.layers:
+        print(f"{'step':44s} {'kind':16s} {'us':>9s}", file=sys.stderr)
+        for label, kind, ms in steps_info:
+            print(f"{label:44s} {kind:16s} {ms * 1e3:9.1f}", file=sys.stderr)
+        print(f"sum of steps (event-bracketed, includes event overhead): {sum_step_ms * 1e3:.1f} us", file=sys.stderr)
+        for row in layer_rows:
+            print("conv %-36s %8.1f us pairs=%8d n_out=%7d bytes=%10d ops=%12d" % row, file=sys.stderr)
+
+    result = {
+        "metric": "frames/s, int8 CenterPoint-shaped SCN backbone @~120k active voxels" if args.precision == "int8"
+                  else "frames/s, fp16 CenterPoint-shaped SCN backbone @~120k active voxels",
+        "value": round(1e3 / ms_per_step, 2), "unit": "frames/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int8" if args.precision == "int8" else "f16", "data": "synthetic",
+        "config": {"workload": "BASELINE.json configs[2]: int8 CenterPoint-shaped SCN backbone, synthetic 250k-point frame"
+                               if args.precision == "int8" else
+                               "BASELINE.json configs[1]: fp16 CenterPoint-shaped SCN backbone, synthetic 250k-point frame",
+                   "points": int(frame.shape[0]), "active_voxels": int(nvox), "grid": list(GRID_ZYX),
+                   "launch": "hip graph replay" if use_graph else "direct launches", "output": out_view.shape},
+        "voxels_per_s": round(nvox * 1e3 / ms_per_step, 1),
+        "voxelization_ms": round(vox_ms, 4),
+        "backbone_gop_per_frame": round(total_ops / 1e9, 2),
+        "backbone_algorithmic_MB_per_frame": round(total_bytes / 1e6, 1),
+        "whole_backbone_TOPs": round(total_ops / (ms_per_step * 1e-3) / 1e12, 3),
+        "whole_backbone_GBs": round(total_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+        "step_us_by_kind": {k: round(v * 1e3, 1) for k, v in by_kind.items()},
+        "layers_us": {label: round(ms * 1e3, 1) for label, kind, ms in steps_info},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "output_checksum": checksum,
+        "setup_s": round(time.perf_counter() - t_setup, 1),
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

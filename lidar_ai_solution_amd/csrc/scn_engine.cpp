@@ -119,7 +119,7 @@ struct RtTensor {
   bool materialised = false;  // false: fused away, never written
 };
 
-enum class StepKind { InputCount, HashBuild, RulebookSubm, RulebookSparse, Convert, Conv, Add, Relu, Dense };
+enum class StepKind { InputCount, HashBuild, RulebookSubm, RulebookSparse, Convert, Conv, Add, Relu, Dense, Permute };
 
 struct Step {
   StepKind kind;
@@ -673,8 +673,37 @@ static bool build_engine(scn_engine& e) {
         break;
       }
       case Op::Transpose: {
-        set_error("node %s: a Transpose that does not directly follow ScatterDense is not supported", n.name.c_str());
-        return false;
+        // reached only when the Transpose was not folded into the preceding ScatterDense
+        RtTensor& x = e.tensors[n.in[0]];
+        if (!x.dense || x.shape.size() != 5 || n.dims.size() != 5) {
+          set_error("node %s: Transpose needs a dense 5-D input and 5 dims", n.name.c_str());
+          return false;
+        }
+        Step st;
+        st.kind = StepKind::Permute;
+        st.node = (int)i;
+        st.label = n.name;
+        st.t_in = n.in[0];
+        st.t_out = n.out;
+        bool seen[5] = {false, false, false, false, false};
+        std::vector<int64_t> shape(5);
+        for (int j = 0; j < 5; ++j) {
+          const int64_t d = n.dims[j];
+          if (d < 0 || d > 4 || seen[d]) {
+            set_error("node %s: dims is not a permutation", n.name.c_str());
+            return false;
+          }
+          seen[d] = true;
+          st.perm[j] = (int)d;
+          shape[j] = x.shape[d];
+        }
+        RtTensor& o = e.tensors[n.out];
+        o.dense = true;
+        o.dtype = x.dtype;
+        o.shape = shape;
+        o.materialised = true;
+        e.steps.push_back(st);
+        break;
       }
     }
   }
@@ -857,6 +886,13 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
       const CoordSet& cs = e.coords[x.coord];
       return scatter_dense(x.data, x.dtype, x.scale, (uint32_t)x.c, x.ld, cs.idx, cs.n_bound, cs.n_dev, st.dense_shape,
                            st.has_perm ? st.perm : nullptr, o.data, stream);
+    }
+    case StepKind::Permute: {
+      const RtTensor& x = e.tensors[st.t_in];
+      RtTensor& o = e.tensors[st.t_out];
+      int64_t shape[5];
+      for (int j = 0; j < 5; ++j) shape[j] = x.shape[j];
+      return permute_dense(x.data, shape, st.perm, o.data, stream);
     }
   }
   return SCN_ERR_INVALID;
@@ -1503,7 +1539,7 @@ int scn_engine_set_profiling(scn_engine* e, int enabled) {
 int scn_engine_num_nodes(const scn_engine* e) { return e ? (int)e->steps.size() : 0; }
 int scn_engine_node_info(scn_engine* e, int node, const char** name, const char** kind, float* last_ms) {
   SCN_REQUIRE(e && node >= 0 && node < (int)e->steps.size(), SCN_ERR_INVALID, "node_info: invalid index");
-  static const char* kinds[] = {"input", "hash", "rulebook_subm", "rulebook_sparse", "convert", "conv", "add", "relu", "dense"};
+  static const char* kinds[] = {"input", "hash", "rulebook_subm", "rulebook_sparse", "convert", "conv", "add", "relu", "dense", "transpose"};
   const Step& s = e->steps[node];
   if (name) *name = s.label.c_str();
   if (kind) *kind = kinds[(int)s.kind];

@@ -1065,6 +1065,48 @@ int scatter_dense(const void* feat, int dtype, float scale, uint32_t c, uint32_t
   return SCN_OK;
 }
 
+// Stand-alone dense permute of a 5-D fp16 tensor (used only when the Transpose is not fused into
+// the scatter): out[o0..o4] = in[index with dim perm[j] = o_j].
+struct Permute5 {
+  int64_t in_stride[5];   // input stride of the dimension that output dim j walks
+  int64_t out_shape[5];
+};
+
+__global__ __launch_bounds__(256) void k_permute5(const _Float16* __restrict__ in, _Float16* out, Permute5 p,
+                                                  size_t numel) {
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= numel) return;
+  size_t rem = i, src = 0;
+#pragma unroll
+  for (int j = 4; j >= 0; --j) {
+    const size_t c = rem % (size_t)p.out_shape[j];
+    rem /= (size_t)p.out_shape[j];
+    src += c * (size_t)p.in_stride[j];
+  }
+  out[i] = in[src];
+}
+
+int permute_dense(const void* in, const int64_t in_shape[5], const int perm[5], void* out, hipStream_t stream) {
+  Permute5 p;
+  int64_t istride[5];
+  int64_t s = 1;
+  for (int j = 4; j >= 0; --j) {
+    istride[j] = s;
+    s *= in_shape[j];
+  }
+  for (int j = 0; j < 5; ++j) {
+    SCN_REQUIRE(perm[j] >= 0 && perm[j] < 5, SCN_ERR_INVALID, "permute: bad permutation");
+    p.in_stride[j] = istride[perm[j]];
+    p.out_shape[j] = in_shape[perm[j]];
+  }
+  const size_t numel = (size_t)s;
+  if (numel == 0) return SCN_OK;
+  hipLaunchKernelGGL(k_permute5, dim3((unsigned)((numel + 255) / 256)), dim3(256), 0, stream, (const _Float16*)in,
+                     (_Float16*)out, p, numel);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
 // --------------------------------------------------------------------------------------------
 // voxelization
 // --------------------------------------------------------------------------------------------

@@ -92,6 +92,8 @@ int add_relu(const void* a, int a_dtype, float a_scale, float a_rq, const void* 
 int scatter_dense(const void* feat, int dtype, float scale, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
                   const uint32_t* n_dev, const int dense_shape[5], const int perm[5], void* out, hipStream_t stream);
 
+int permute_dense(const void* in, const int64_t in_shape[5], const int perm[5], void* out, hipStream_t stream);
+
 }  // namespace scn
 
 // Voxelizer object of the C ABI.
