@@ -13,6 +13,7 @@
 #include "scn_kernels.hpp"
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <type_traits>
 #include <vector>
@@ -232,45 +233,51 @@ __global__ __launch_bounds__(1024) void k_scan_blocksums(uint32_t* vals, uint32_
   }
 }
 
-// Expands the set bits in rank order.  Optional outputs: coordinate rows, a hash table of
-// {key -> rank}, and the per-word exclusive prefix (rank of the word's first bit).
-__global__ __launch_bounds__(256) void k_bitmap_expand(const uint32_t* __restrict__ bitmap,
-                                                       const uint32_t* __restrict__ blockoff, Int3 grid, uint32_t cap,
-                                                       int4* coords_out, uint64_t* slots, uint32_t mask,
-                                                       uint32_t* prefix_out) {
+// Sparse bitmaps (fewer set bits than words): one thread per word expands its bits in rank order.
+// Optional outputs: coordinate rows, a hash table of {key -> rank}, and the per-word exclusive
+// prefix (rank of the word's first bit).  Block = 1024 threads = 1024 words.
+__global__ __launch_bounds__(1024) void k_bitmap_expand(const uint32_t* __restrict__ bitmap,
+                                                        const uint32_t* __restrict__ blockoff, Int3 grid, uint32_t cap,
+                                                        int4* coords_out, uint64_t* slots, uint32_t mask,
+                                                        uint32_t* prefix_out) {
   __shared__ uint32_t scratch[17];
-  const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
-  const uint4 w4 = reinterpret_cast<const uint4*>(bitmap)[t];
-  const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
-  const uint32_t c = __popc(w[0]) + __popc(w[1]) + __popc(w[2]) + __popc(w[3]);
+  const size_t t = (size_t)blockIdx.x * 1024 + threadIdx.x;
+  uint32_t bits = bitmap[t];
+  const uint32_t c = __popc(bits);
   uint32_t total;
   uint32_t rank = blockoff[blockIdx.x] + block_exclusive_scan(c, scratch, &total);
-  if (prefix_out) {
-    uint4 p;
-    p.x = rank;
-    p.y = p.x + __popc(w[0]);
-    p.z = p.y + __popc(w[1]);
-    p.w = p.z + __popc(w[2]);
-    reinterpret_cast<uint4*>(prefix_out)[t] = p;
-  }
+  if (prefix_out) prefix_out[t] = rank;
   if (c == 0 || coords_out == nullptr) return;
   const uint32_t g12 = (uint32_t)grid.v[1] * (uint32_t)grid.v[2];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    uint32_t bits = w[j];
-    while (bits) {
-      const int b = __ffs(bits) - 1;
-      bits &= bits - 1;
-      if (rank < cap) {
-        const uint32_t key = (uint32_t)(t * 4 + j) * 32u + (uint32_t)b;
-        const uint32_t i0 = key / g12, rem = key - i0 * g12;
-        const uint32_t i1 = rem / (uint32_t)grid.v[2], i2 = rem - i1 * (uint32_t)grid.v[2];
-        coords_out[rank] = make_int4(0, (int)i0, (int)i1, (int)i2);
-        if (slots) table_insert(slots, mask, key, rank);
-      }
-      rank++;
+  while (bits) {
+    const int b = __ffs(bits) - 1;
+    bits &= bits - 1;
+    if (rank < cap) {
+      const uint32_t key = (uint32_t)t * 32u + (uint32_t)b;
+      const uint32_t i0 = key / g12, rem = key - i0 * g12;
+      const uint32_t i1 = rem / (uint32_t)grid.v[2], i2 = rem - i1 * (uint32_t)grid.v[2];
+      coords_out[rank] = make_int4(0, (int)i0, (int)i1, (int)i2);
+      if (slots) table_insert(slots, mask, key, rank);
     }
+    rank++;
   }
+}
+
+// Dense bitmaps: one thread per cell, rank = prefix of its word + set bits below it.
+__global__ __launch_bounds__(256) void k_expand_cells(const uint32_t* __restrict__ bitmap,
+                                                      const uint32_t* __restrict__ prefix, uint32_t cells, Int3 grid,
+                                                      uint32_t cap, int4* coords_out, uint64_t* slots, uint32_t mask) {
+  const uint32_t key = blockIdx.x * 256 + threadIdx.x;
+  if (key >= cells) return;
+  const uint32_t w = bitmap[key >> 5], b = key & 31;
+  if (!((w >> b) & 1u)) return;
+  const uint32_t rank = prefix[key >> 5] + __popc(w & ((1u << b) - 1u));
+  if (rank >= cap) return;
+  const uint32_t g12 = (uint32_t)grid.v[1] * (uint32_t)grid.v[2];
+  const uint32_t i0 = key / g12, rem = key - i0 * g12;
+  const uint32_t i1 = rem / (uint32_t)grid.v[2], i2 = rem - i1 * (uint32_t)grid.v[2];
+  coords_out[rank] = make_int4(0, (int)i0, (int)i1, (int)i2);
+  if (slots) table_insert(slots, mask, key, rank);
 }
 
 static size_t bitmap_words_for(const int g[3]) {
@@ -299,7 +306,8 @@ static GeomDev to_dev(const ConvGeom& g) {
   return d;
 }
 
-// nbr[k][o] = row of the input at  o*stride - pad + k*dilation  (or -1).  grid.y = kernel offset.
+// nbr[k][o] = row of the input at  o*stride - pad + k*dilation  (or -1).  grid.y = k0; a thread
+// walks the K1*K2 offsets of its k0 plane (independent lookups, coalesced stores per offset).
 // Used for both kinds: submanifold passes stride 1 and pad = floor(K/2)*dilation.
 __global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_coords, const uint32_t* n_out_dev,
                                                    uint32_t n_bound, GeomDev g, const uint64_t* __restrict__ slots,
@@ -307,43 +315,60 @@ __global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_
   const uint32_t n = eff_n(n_out_dev, n_bound);
   const uint32_t o = blockIdx.x * 256 + threadIdx.x;
   if (o >= n) return;
-  const int k = blockIdx.y;
-  const int k2 = k % g.ks[2], k1 = (k / g.ks[2]) % g.ks[1], k0 = k / (g.ks[2] * g.ks[1]);
+  const int k0 = blockIdx.y;
   const int4 c = out_coords[o];
-  int32_t res = -1;
-  if (identity_center && k0 == g.ks[0] / 2 && k1 == g.ks[1] / 2 && k2 == g.ks[2] / 2) {
-    res = (int32_t)o;
-  } else {
-    const int i0 = c.y * g.st[0] - g.pd[0] + k0 * g.dl[0];
+  const int i0 = c.y * g.st[0] - g.pd[0] + k0 * g.dl[0];
+  const bool ok0 = c.x == 0 && i0 >= 0 && i0 < g.gi[0];
+  const bool centre0 = identity_center && k0 == g.ks[0] / 2;
+  for (int k1 = 0; k1 < g.ks[1]; ++k1) {
     const int i1 = c.z * g.st[1] - g.pd[1] + k1 * g.dl[1];
-    const int i2 = c.w * g.st[2] - g.pd[2] + k2 * g.dl[2];
-    if (c.x == 0 && i0 >= 0 && i0 < g.gi[0] && i1 >= 0 && i1 < g.gi[1] && i2 >= 0 && i2 < g.gi[2]) {
-      const uint32_t key = ((uint32_t)i0 * (uint32_t)g.gi[1] + (uint32_t)i1) * (uint32_t)g.gi[2] + (uint32_t)i2;
-      res = table_lookup(slots, mask, key);
+    const bool ok1 = ok0 && i1 >= 0 && i1 < g.gi[1];
+#pragma unroll 3
+    for (int k2 = 0; k2 < g.ks[2]; ++k2) {
+      const int i2 = c.w * g.st[2] - g.pd[2] + k2 * g.dl[2];
+      int32_t res = -1;
+      if (centre0 && k1 == g.ks[1] / 2 && k2 == g.ks[2] / 2) {
+        res = (int32_t)o;
+      } else if (ok1 && i2 >= 0 && i2 < g.gi[2]) {
+        const uint32_t key = ((uint32_t)i0 * (uint32_t)g.gi[1] + (uint32_t)i1) * (uint32_t)g.gi[2] + (uint32_t)i2;
+        res = table_lookup(slots, mask, key);
+      }
+      nbr[(size_t)((k0 * g.ks[1] + k1) * g.ks[2] + k2) * ld + o] = res;
     }
   }
-  nbr[(size_t)k * ld + o] = res;
 }
 
-// Marks every output cell reached by an input row through some kernel offset.  grid.y = offset.
+// Marks every output cell reached by an input row through some kernel offset.  One thread per
+// input row; the bit is tested before the atomic so that cells reached by several inputs cost one
+// atomic, not one per input.
 __global__ __launch_bounds__(256) void k_mark_outputs(const int4* __restrict__ in_coords, const uint32_t* n_dev,
                                                       uint32_t n_bound, GeomDev g, uint32_t* bitmap) {
   const uint32_t n = eff_n(n_dev, n_bound);
   const uint32_t r = blockIdx.x * 256 + threadIdx.x;
   if (r >= n) return;
-  const int k = blockIdx.y;
-  const int k2 = k % g.ks[2], k1 = (k / g.ks[2]) % g.ks[1], k0 = k / (g.ks[2] * g.ks[1]);
   const int4 c = in_coords[r];
   if (c.x != 0 || c.y < 0 || c.y >= g.gi[0] || c.z < 0 || c.z >= g.gi[1] || c.w < 0 || c.w >= g.gi[2]) return;
-  const int t0 = c.y + g.pd[0] - k0 * g.dl[0];
-  const int t1 = c.z + g.pd[1] - k1 * g.dl[1];
-  const int t2 = c.w + g.pd[2] - k2 * g.dl[2];
-  if (t0 < 0 || t1 < 0 || t2 < 0) return;
-  if (t0 % g.st[0] || t1 % g.st[1] || t2 % g.st[2]) return;
-  const int o0 = t0 / g.st[0], o1 = t1 / g.st[1], o2 = t2 / g.st[2];
-  if (o0 >= g.go[0] || o1 >= g.go[1] || o2 >= g.go[2]) return;
-  const uint32_t key = ((uint32_t)o0 * (uint32_t)g.go[1] + (uint32_t)o1) * (uint32_t)g.go[2] + (uint32_t)o2;
-  atomicOr(&bitmap[key >> 5], 1u << (key & 31));
+  for (int k0 = 0; k0 < g.ks[0]; ++k0) {
+    const int t0 = c.y + g.pd[0] - k0 * g.dl[0];
+    if (t0 < 0 || t0 % g.st[0]) continue;
+    const int o0 = t0 / g.st[0];
+    if (o0 >= g.go[0]) continue;
+    for (int k1 = 0; k1 < g.ks[1]; ++k1) {
+      const int t1 = c.z + g.pd[1] - k1 * g.dl[1];
+      if (t1 < 0 || t1 % g.st[1]) continue;
+      const int o1 = t1 / g.st[1];
+      if (o1 >= g.go[1]) continue;
+      for (int k2 = 0; k2 < g.ks[2]; ++k2) {
+        const int t2 = c.w + g.pd[2] - k2 * g.dl[2];
+        if (t2 < 0 || t2 % g.st[2]) continue;
+        const int o2 = t2 / g.st[2];
+        if (o2 >= g.go[2]) continue;
+        const uint32_t key = ((uint32_t)o0 * (uint32_t)g.go[1] + (uint32_t)o1) * (uint32_t)g.go[2] + (uint32_t)o2;
+        const uint32_t bit = 1u << (key & 31);
+        if (!(bitmap[key >> 5] & bit)) atomicOr(&bitmap[key >> 5], bit);
+      }
+    }
+  }
 }
 
 bool Rulebook::init(uint32_t max_in_, uint32_t max_out_, int kvol) {
@@ -384,7 +409,7 @@ int set_count(uint32_t* dst, const uint32_t* n_dev, uint32_t n_bound, hipStream_
 static int launch_build_nbr(const Rulebook& rb, const int32_t* out_coords, uint32_t n_bound, bool identity_center,
                             hipStream_t stream) {
   if (n_bound == 0) return SCN_OK;
-  hipLaunchKernelGGL(k_build_nbr, dim3(ceil_div(n_bound, 256), rb.geom.kvol), dim3(256), 0, stream,
+  hipLaunchKernelGGL(k_build_nbr, dim3(ceil_div(n_bound, 256), rb.geom.ks[0]), dim3(256), 0, stream,
                      (const int4*)out_coords, rb.n_out_dev(), n_bound, to_dev(rb.geom), rb.in_table->slots(),
                      rb.in_table->mask, rb.nbr.as<int32_t>(), rb.ld, identity_center ? 1 : 0);
   SCN_HIP(hipGetLastError());
@@ -461,6 +486,7 @@ int Rulebook::build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev
   if (words != bitmap_words) {
     if (!bitmap.alloc(words * 4)) return SCN_ERR_HIP;
     if (!blocksum.alloc((words / kWordsPerBlock + 1) * 4)) return SCN_ERR_HIP;
+    if (!prefix.alloc(words * 4)) return SCN_ERR_HIP;
     bitmap_words = words;
   }
   if (out_idx.bytes < (size_t)max_out * 16 && !out_idx.alloc((size_t)std::max(max_out, 1u) * 16)) return SCN_ERR_HIP;
@@ -484,7 +510,7 @@ int Rulebook::build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev
   if (rc) return rc;
   const GeomDev gd = to_dev(geom);
   if (n) {
-    hipLaunchKernelGGL(k_mark_outputs, dim3(ceil_div(n, 256), geom.kvol), dim3(256), 0, stream, (const int4*)idx,
+    hipLaunchKernelGGL(k_mark_outputs, dim3(ceil_div(n, 256)), dim3(256), 0, stream, (const int4*)idx,
                        n_dev, n, gd, bitmap.as<uint32_t>());
   }
   const uint32_t nblocks = (uint32_t)(words / kWordsPerBlock);
@@ -492,9 +518,21 @@ int Rulebook::build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev
                      blocksum.as<uint32_t>());
   hipLaunchKernelGGL(k_scan_blocksums, dim3(1), dim3(1024), 0, stream, blocksum.as<uint32_t>(), nblocks, cnt,
                      n_bound_out);
-  hipLaunchKernelGGL(k_bitmap_expand, dim3(nblocks), dim3(256), 0, stream, bitmap.as<uint32_t>(),
-                     blocksum.as<uint32_t>(), Int3{{geom.grid_out[0], geom.grid_out[1], geom.grid_out[2]}},
-                     n_bound_out, (int4*)out_idx.p, out_table.slots(), out_table.mask, (uint32_t*)nullptr);
+  const Int3 og{{geom.grid_out[0], geom.grid_out[1], geom.grid_out[2]}};
+  const uint64_t cells = (uint64_t)geom.grid_out[0] * geom.grid_out[1] * geom.grid_out[2];
+  if (cells <= 32ull * std::max(n_bound_out, 1u)) {
+    // dense output grid: per-word prefix, then one thread per cell
+    hipLaunchKernelGGL(k_bitmap_expand, dim3(nblocks), dim3(1024), 0, stream, bitmap.as<uint32_t>(),
+                       blocksum.as<uint32_t>(), og, n_bound_out, (int4*)nullptr, (uint64_t*)nullptr, 0u,
+                       prefix.as<uint32_t>());
+    hipLaunchKernelGGL(k_expand_cells, dim3((unsigned)((cells + 255) / 256)), dim3(256), 0, stream,
+                       bitmap.as<uint32_t>(), prefix.as<uint32_t>(), (uint32_t)cells, og, n_bound_out, (int4*)out_idx.p,
+                       out_table.slots(), out_table.mask);
+  } else {
+    hipLaunchKernelGGL(k_bitmap_expand, dim3(nblocks), dim3(1024), 0, stream, bitmap.as<uint32_t>(),
+                       blocksum.as<uint32_t>(), og, n_bound_out, (int4*)out_idx.p, out_table.slots(), out_table.mask,
+                       (uint32_t*)nullptr);
+  }
   SCN_HIP(hipGetLastError());
   rc = launch_build_nbr(*this, out_indices, n_bound_out, false, stream);
   if (rc) return rc;
@@ -605,6 +643,7 @@ struct ConvArgs {
   float mid_scale;
   float a_rq, b_rq;
   int relu2;
+  int debug;  // measurement knob: 1 = no gathers, 2 = no weight slab loads, 8 = no epilogue, 16 = no main loop
 };
 
 __device__ __forceinline__ float quant_f(float y, float s) {
@@ -620,6 +659,9 @@ struct Mma;
 template <>
 struct Mma<0> {
   using Acc = v4i;
+  static __device__ __forceinline__ Acc run(const v4i a, const v4i b, Acc c) {
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+  }
   static __device__ __forceinline__ Acc run(const uint4& a, const uint4& b, Acc c) {
     return __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, a), __builtin_bit_cast(v4i, b), c, 0, 0, 0);
   }
@@ -627,10 +669,25 @@ struct Mma<0> {
 template <>
 struct Mma<1> {
   using Acc = v4f;
+  static __device__ __forceinline__ Acc run(const v4i a, const v4i b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
   static __device__ __forceinline__ Acc run(const uint4& a, const uint4& b, Acc c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
   }
 };
+
+// Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2.  Giving XCD x the
+// x-th contiguous eighth of the row tiles keeps the rows a tile gathers (spatial neighbours, i.e.
+// nearby rows in canonical order) inside one L2 instead of spreading every row over all eight.
+// Returns false when this workgroup has no tile.
+__device__ __forceinline__ bool xcd_tile(uint32_t n, uint32_t rows_per_block, uint32_t* tile) {
+  const uint32_t tiles = (n + rows_per_block - 1) / rows_per_block;
+  const uint32_t per = (tiles + 7) >> 3;
+  const uint32_t xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+  *tile = xcd * per + j;
+  return j < per && *tile < tiles;
+}
 
 // Stores 4 consecutive channels of one row after the fused epilogue.
 template <int EL>
@@ -714,7 +771,9 @@ __global__ __launch_bounds__(256) void k_conv_rows(const ConvArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int lr = lane & 15, lg = lane >> 4;
   const uint32_t n = eff_n(a.n_out_dev, a.n_bound);
-  const uint32_t row0 = (blockIdx.x * 4 + wave) * (16 * NT);
+  uint32_t tile;
+  if (!xcd_tile(n, 64u * NT, &tile)) return;
+  const uint32_t row0 = (tile * 4 + wave) * (16 * NT);
   if (row0 >= n) return;
   Acc acc[MT][NT];
 #pragma unroll
@@ -742,10 +801,11 @@ __global__ __launch_bounds__(256) void k_conv_rows(const ConvArgs a) {
       for (int ss = 0; ss < SPK; ++ss) {
         uint4 b[NT];
 #pragma unroll
-        for (int u = 0; u < NT; ++u)
-          b[u] = idx[u] >= 0
-                     ? *reinterpret_cast<const uint4*>(a.x + (size_t)idx[u] * a.x_ld_bytes + (ss * 4 + lg) * 16)
-                     : zero;
+        for (int u = 0; u < NT; ++u) {
+          b[u] = *reinterpret_cast<const uint4*>(a.x + (size_t)(idx[u] >= 0 ? idx[u] : 0) * a.x_ld_bytes +
+                                                 (ss * 4 + lg) * 16);
+          if (idx[u] < 0) b[u] = zero;
+        }
         const int s = k * SPK + ss;
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
@@ -768,7 +828,8 @@ __global__ __launch_bounds__(256) void k_conv_rows(const ConvArgs a) {
         int32_t idx = -1;
         if (gv && rows[u] < n) idx = a.nbr[(size_t)k * a.nbr_ld + rows[u]];
         any |= idx >= 0;
-        b[u] = idx >= 0 ? *reinterpret_cast<const uint4*>(a.x + (size_t)idx * a.x_ld_bytes + c * 16) : zero;
+        b[u] = *reinterpret_cast<const uint4*>(a.x + (size_t)(idx >= 0 ? idx : 0) * a.x_ld_bytes + c * 16);
+        if (idx < 0) b[u] = zero;
       }
       if (!__any(any)) continue;
 #pragma unroll
@@ -782,6 +843,174 @@ __global__ __launch_bounds__(256) void k_conv_rows(const ConvArgs a) {
 #pragma unroll
   for (int u = 0; u < NT; ++u) {
     if (rows[u] >= n) continue;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) epilogue_store<EL>(a, rows[u], t * 16 + lg * 4, acc[t][u]);
+  }
+}
+
+constexpr int kConvMaxKvol = 27;  // largest kernel volume the workgroup kernel keeps in LDS
+
+// Workgroup kernel: 4 waves, each owning 16*NT output rows and all MT*16 output channels.
+//   * the weight slab of one iteration (one kernel offset when a row has >= 4 chunks, else 4/CHUNKS
+//     offsets) is staged through LDS once per workgroup, double-buffered, and read back as MFMA A
+//     fragments with ds_read_b128 (its own wait counter, so it never blocks on the gathers);
+//   * gathered rows go from global memory straight into the MFMA B operand, one iteration ahead;
+//   * neighbour indices are fetched two iterations ahead.
+// So during the MFMAs of iteration i the gathers and the weight slab of i+1 and the indices of i+2
+// are in flight.  Loaded values are only touched (masked, stored) in the iteration that consumes
+// them: any earlier ALU use would make the wave wait for the load right where it was issued.
+template <int EL, int CHUNKS, int MT, int NT>
+__global__ __launch_bounds__(256) void k_conv_wg(const ConvArgs a) {
+  using Acc = typename Mma<EL>::Acc;
+  constexpr int SPK = CHUNKS >= 4 ? CHUNKS / 4 : 1;  // K-steps per iteration
+  constexpr int SLAB = SPK * MT * 64;                 // 16-byte fragments per iteration
+  constexpr int WPT = (SLAB + 255) / 256;             // fragments staged per thread
+  constexpr int R = 64 * NT;                          // output rows per workgroup
+  __shared__ v4i lds[2][SLAB];
+  __shared__ int32_t lidx[kConvMaxKvol * R];          // neighbour rows of the whole tile, all offsets
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const uint32_t n = eff_n(a.n_out_dev, a.n_bound);
+  uint32_t tile;
+  if (!xcd_tile(n, 64u * NT, &tile)) return;  // uniform for the whole workgroup
+  const uint32_t row0 = (tile * 4 + wave) * (16 * NT);
+  // The neighbour table is read exactly once, so every one of its loads misses the caches.  Fetch the
+  // tile's whole block (kvol x R indices) up front with all loads in flight together, instead of
+  // paying that latency once per kernel offset inside the pipelined loop.
+  {
+    const uint32_t tile_row0 = tile * R;
+    const int total = a.kvol * R;
+    for (int base = 0; base < total; base += 256 * 8) {
+      int32_t tmp[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int f = base + j * 256 + tid;
+        const int k = f / R, r = f - k * R;
+        const bool v = f < total && tile_row0 + r < n;
+        tmp[j] = v ? a.nbr[(size_t)k * a.nbr_ld + tile_row0 + r] : -1;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int f = base + j * 256 + tid;
+        if (f < total) lidx[f] = tmp[j];
+      }
+    }
+  }
+  __syncthreads();
+  const int32_t* __restrict__ my_idx = lidx + wave * (16 * NT) + lr;
+  const int iters = CHUNKS >= 4 ? a.kvol : a.steps;
+  const int total_chunks = a.kvol * CHUNKS;
+  const char* __restrict__ xb = a.x;
+  const v4i* __restrict__ wsrc = reinterpret_cast<const v4i*>(a.wfrag);
+  const uint32_t ldb = a.x_ld_bytes;
+  uint32_t rows[NT];
+  bool rvalid[NT];
+#pragma unroll
+  for (int u = 0; u < NT; ++u) {
+    rows[u] = row0 + u * 16 + lr;
+    rvalid[u] = rows[u] < n;
+  }
+
+  Acc acc[MT][NT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int u = 0; u < NT; ++u) acc[t][u] = Acc{0, 0, 0, 0};
+
+  int32_t idx0[NT], idx1[NT], idx2[NT];
+  v4i bcur[SPK][NT], bnext[SPK][NT];
+  v4i wreg[WPT];
+  const v4i vzero = {0, 0, 0, 0};
+
+// does this lane's slot of iteration IT exist at all (known without any load)
+#define SCN_SLOT_VALID(IT) ((IT) < iters && (CHUNKS >= 4 || 4 * (IT) + lg < total_chunks))
+#define SCN_SLOT_K(IT) (CHUNKS >= 4 ? (IT) : (4 * (IT) + lg) / CHUNKS)
+// neighbour indices of iteration IT from the LDS copy (rows beyond n hold -1 there)
+#define SCN_LOAD_IDX(IT, DST)                                                 \
+  {                                                                           \
+    const int k_ = SCN_SLOT_VALID(IT) ? SCN_SLOT_K(IT) : 0;                   \
+    _Pragma("unroll") for (int u = 0; u < NT; ++u) DST[u] = my_idx[k_ * R + u * 16]; \
+  }
+// unconditional gathers (row 0 for lanes without a neighbour); masked to zero when consumed
+#define SCN_GATHER(IT, IDX, DST)                                                            \
+  {                                                                                         \
+    const bool sv_ = SCN_SLOT_VALID(IT);                                                    \
+    _Pragma("unroll") for (int u = 0; u < NT; ++u) {                                        \
+      const bool ok_ = sv_ && rvalid[u] && IDX[u] >= 0;                                     \
+      const char* p_ = xb + (size_t)(ok_ ? (uint32_t)IDX[u] : 0u) * ldb;                    \
+      _Pragma("unroll") for (int ss = 0; ss < SPK; ++ss) {                                  \
+        const int c_ = CHUNKS >= 4 ? ss * 4 + lg : (4 * (IT) + lg) % CHUNKS;                \
+        DST[ss][u] = *reinterpret_cast<const v4i*>(p_ + c_ * 16);                           \
+      }                                                                                     \
+    }                                                                                       \
+  }
+#define SCN_LOAD_SLAB(IT)                                                     \
+  {                                                                           \
+    _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                         \
+      const int f_ = tid + j * 256;                                           \
+      if (SLAB % 256 == 0 || f_ < SLAB) wreg[j] = wsrc[(size_t)(IT) * SLAB + f_]; \
+    }                                                                         \
+  }
+#define SCN_STORE_SLAB(BUF)                                                   \
+  {                                                                           \
+    _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                         \
+      const int f_ = tid + j * 256;                                           \
+      if (SLAB % 256 == 0 || f_ < SLAB) lds[BUF][f_] = wreg[j];               \
+    }                                                                         \
+  }
+
+  SCN_LOAD_IDX(0, idx0);
+  SCN_LOAD_IDX(1, idx1);
+  SCN_LOAD_SLAB(0);
+  SCN_GATHER(0, idx0, bcur);
+  SCN_STORE_SLAB(0);
+  __syncthreads();
+  for (int it = 0; it < ((a.debug & 16) ? 0 : iters); ++it) {
+    SCN_LOAD_IDX(it + 2, idx2);
+    const bool more = it + 1 < iters;
+    if (more) {
+      if (!(a.debug & 2)) SCN_LOAD_SLAB(it + 1);
+      if (!(a.debug & 1)) SCN_GATHER(it + 1, idx1, bnext);
+    }
+    // MFMAs are unconditional: a branch around them makes the compiler shuttle all accumulators
+    // between AGPRs and VGPRs every iteration, which costs far more than multiplying by zero.
+    {
+      const bool sv = SCN_SLOT_VALID(it);
+      const v4i* la = lds[it & 1] + lane;
+#pragma unroll
+      for (int ss = 0; ss < SPK; ++ss) {
+        v4i bm[NT];
+#pragma unroll
+        for (int u = 0; u < NT; ++u) bm[u] = (sv && rvalid[u] && idx0[u] >= 0) ? bcur[ss][u] : vzero;
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          const v4i av = la[(ss * MT + t) * 64];
+#pragma unroll
+          for (int u = 0; u < NT; ++u) acc[t][u] = Mma<EL>::run(av, bm[u], acc[t][u]);
+        }
+      }
+    }
+    if (more) SCN_STORE_SLAB((it + 1) & 1);
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < NT; ++u) {
+      idx0[u] = idx1[u];
+      idx1[u] = idx2[u];
+#pragma unroll
+      for (int ss = 0; ss < SPK; ++ss) bcur[ss][u] = bnext[ss][u];
+    }
+  }
+#undef SCN_SLOT_VALID
+#undef SCN_SLOT_K
+#undef SCN_LOAD_IDX
+#undef SCN_GATHER
+#undef SCN_LOAD_SLAB
+#undef SCN_STORE_SLAB
+  if (a.debug & 8) return;
+#pragma unroll
+  for (int u = 0; u < NT; ++u) {
+    if (!rvalid[u]) continue;
 #pragma unroll
     for (int t = 0; t < MT; ++t) epilogue_store<EL>(a, rows[u], t * 16 + lg * 4, acc[t][u]);
   }
@@ -852,12 +1081,32 @@ bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* 
   return true;
 }
 
+// 0: workgroup kernel (LDS-staged weights, software-pipelined gathers); 1: plain row-split kernel.
+// The second is kept for A/B measurements (environment variable SCN_CONV_IMPL=rows).
+static int conv_impl() {
+  static const int impl = [] {
+    const char* e = getenv("SCN_CONV_IMPL");
+    return (e && !strcmp(e, "rows")) ? 1 : 0;
+  }();
+  return impl;
+}
+
 template <int EL, int CHUNKS, int MT>
 static void launch_conv_rows(const ConvArgs& a, hipStream_t stream) {
+  // Row tiles per wave.  4 for up to 64 output channels; 2 for 128: with 4 the accumulators alone take
+  // 128 registers, occupancy drops to one workgroup per CU and a 65 k-row layer becomes 257 workgroups
+  // on 256 CUs (measured 127 us against 62 us).
   constexpr int NT = MT >= 8 ? 2 : 4;
   const uint32_t rows_per_block = 4 * 16 * NT;
-  hipLaunchKernelGGL((k_conv_rows<EL, CHUNKS, MT, NT>), dim3(ceil_div(a.n_bound, rows_per_block)), dim3(256), 0, stream,
-                     a);
+  constexpr int SPK = CHUNKS >= 4 ? CHUNKS / 4 : 1;
+  constexpr bool lds_ok = 2 * SPK * MT * 64 * 16 + kConvMaxKvol * 64 * NT * 4 <= 64 * 1024;
+  const uint32_t blocks = 8 * ceil_div(ceil_div(a.n_bound, rows_per_block), 8);  // see xcd_tile()
+  if (conv_impl() == 0 && lds_ok && a.kvol <= kConvMaxKvol) {
+    if constexpr (lds_ok)
+      hipLaunchKernelGGL((k_conv_wg<EL, CHUNKS, MT, NT>), dim3(blocks), dim3(256), 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((k_conv_rows<EL, CHUNKS, MT, NT>), dim3(blocks), dim3(256), 0, stream, a);
+  }
 }
 
 template <int EL, int CHUNKS>
@@ -934,6 +1183,10 @@ int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, cons
   a.a_rq = io.a_requant_scale;
   a.b_rq = io.b_requant_scale;
   a.relu2 = io.relu_after_add;
+  {
+    static const int dbg = getenv("SCN_CONV_DEBUG") ? atoi(getenv("SCN_CONV_DEBUG")) : 0;
+    a.debug = dbg;
+  }
   bool ok = w.precision == SCN_PRECISION_INT8 ? dispatch_chunks<0>(w.chunks, w.mtiles, a, stream)
                                                : dispatch_chunks<1>(w.chunks, w.mtiles, a, stream);
   SCN_REQUIRE(ok, SCN_ERR_UNSUPPORTED, "conv: no kernel for Cin=%d Cout=%d (chunks %d, m-tiles %d)", w.cin, w.cout,
@@ -1308,7 +1561,7 @@ int scn_voxelizer_forward(scn_voxelizer* v, const void* points_fp16_dev, uint32_
                      v->blocksum.as<uint32_t>());
   hipLaunchKernelGGL(k_scan_blocksums, dim3(1), dim3(1024), 0, stream, v->blocksum.as<uint32_t>(), nblocks, cnt,
                      (uint32_t)p.max_voxels);
-  hipLaunchKernelGGL(k_bitmap_expand, dim3(nblocks), dim3(256), 0, stream, v->bitmap.as<uint32_t>(),
+  hipLaunchKernelGGL(k_bitmap_expand, dim3(nblocks), dim3(1024), 0, stream, v->bitmap.as<uint32_t>(),
                      v->blocksum.as<uint32_t>(), Int3{{g.og[0], g.og[1], g.og[2]}}, (uint32_t)p.max_voxels,
                      (int4*)v->idx.p, (uint64_t*)nullptr, 0u, v->prefix.as<uint32_t>());
   if (num_points) {

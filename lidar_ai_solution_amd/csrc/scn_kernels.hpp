@@ -41,7 +41,7 @@ struct Rulebook {
   uint32_t ld = 0;
   DevBuf out_idx;             // int32 [max_out][4] (strided)
   DevBuf counters;            // uint32: [0] n_out kept, [1] n_out before truncation, [2..] scratch
-  DevBuf bitmap, blocksum;    // strided: occupancy bitmap of the output grid + per-block popcounts
+  DevBuf bitmap, blocksum, prefix;  // strided: occupancy bitmap of the output grid, per-block popcounts, per-word ranks
   size_t bitmap_words = 0;
   DevBuf pair_scratch;        // pair compaction: per (k, block) counts
   const int32_t* in_indices = nullptr;
