@@ -30,17 +30,17 @@ class VoxelizationParam(C.Structure):
 
 
 class ConvIO(C.Structure):
-    _fields_ = [("x_dev", vp), ("x_ld", u32), ("x_scale", C.c_float), ("relu", C.c_int), ("out_dtype", C.c_int),
-                ("out_scale", C.c_float), ("out_dev", vp), ("out_ld", u32), ("acc_dev", vp), ("res_dev", vp),
-                ("res_dtype", C.c_int), ("res_scale", C.c_float), ("res_ld", u32), ("mid_dtype", C.c_int),
-                ("mid_scale", C.c_float), ("a_requant_scale", C.c_float), ("b_requant_scale", C.c_float),
+    _fields_ = [("x_dev", vp), ("x_ld", u32), ("x_dynamic_range", C.c_float), ("relu", C.c_int), ("out_dtype", C.c_int),
+                ("out_dynamic_range", C.c_float), ("out_dev", vp), ("out_ld", u32), ("acc_dev", vp), ("res_dev", vp),
+                ("res_dtype", C.c_int), ("res_dynamic_range", C.c_float), ("res_ld", u32), ("mid_dtype", C.c_int),
+                ("mid_dynamic_range", C.c_float), ("a_requant_range", C.c_float), ("b_requant_range", C.c_float),
                 ("relu_after_add", C.c_int)]
 
 
 class TensorView(C.Structure):
     _fields_ = [("name", C.c_char_p), ("features_dev", vp), ("dtype", C.c_int), ("ndim", C.c_int),
                 ("shape", C.c_int64 * 8), ("indices_dev", vp), ("num_dev", vp), ("grid_size", C.c_int * 3),
-                ("scale", C.c_float)]
+                ("dynamic_range", C.c_float)]
 
 
 LOG_CALLBACK = C.CFUNCTYPE(None, C.c_char_p, C.c_int, C.c_char_p, C.c_int, vp)
@@ -104,6 +104,7 @@ _SIGNATURES = {
     "scn_engine_num_output": (C.c_int, [vp]),
     "scn_engine_set_input": (C.c_int, [vp, C.c_int, vp, u32, u32, vp, i3]),
     "scn_engine_set_num_points_device_ptr": (C.c_int, [vp, C.c_int, vp]),
+    "scn_engine_prepare": (C.c_int, [vp, i3]),
     "scn_engine_forward": (C.c_int, [vp, vp]),
     "scn_engine_output": (C.c_int, [vp, C.c_int, C.POINTER(TensorView)]),
     "scn_engine_tensor": (C.c_int, [vp, C.c_char_p, C.POINTER(TensorView), C.POINTER(vp)]),

@@ -107,7 +107,7 @@ struct CoordSet {
 struct RtTensor {
   bool dense = false;
   int dtype = SCN_DTYPE_FP16;
-  float scale = 1.f;   // int8: value = q * scale
+  float range = 0.f;   // int8: dynamic range (amax); value = q * (range / 127)
   int c = 0;           // logical channels
   uint32_t ld = 0;     // row stride in elements
   int coord = -1;      // CoordSet index (sparse)
@@ -132,14 +132,14 @@ struct Step {
   int conv = -1;
   // convert
   int cv_dtype = 0;
-  float cv_scale = 1.f;
+  float cv_range = 0.f;
   uint32_t cv_c = 0;
   int relu = 0;
   // conv epilogue
-  float x_scale = 1.f;
+  float x_range = 0.f;
   bool fused_add = false;
   int mid_dtype = 0;
-  float mid_scale = 1.f, a_rq = 0.f, b_rq = 0.f;
+  float mid_range = 0.f, a_rq = 0.f, b_rq = 0.f;  // dynamic ranges
   int relu2 = 0;
   bool conv_input_is_converted = false;
   int t_conv_in = -1;  // tensor or conversion buffer index actually read
@@ -204,7 +204,7 @@ namespace scn {
 // ---------------------------------------------------------------------------------------------
 struct Plan {
   std::vector<int> comp, outp;             // per node effective precisions
-  std::vector<float> scale;                // per tensor, <= 0 when no consumer fixes one
+  std::vector<float> range;                // per tensor dynamic range, <= 0 when no consumer fixes one
   std::vector<std::vector<std::pair<int, int>>> consumers;  // per tensor: (node, slot)
 };
 
@@ -231,18 +231,18 @@ static Plan make_plan(const std::vector<NodeDesc>& nodes, size_t ntensors, int e
       p.outp[i] = n.out_precision == SCN_PRECISION_INT8 ? SCN_PRECISION_INT8 : SCN_PRECISION_FP16;
     }
   }
-  // scale of a tensor = what its consumers expect: int8 conv first, then through Relu, then int8 Add,
+  // dynamic range of a tensor = what its consumers expect: int8 conv first, then through Relu, then int8 Add,
   // then an int8 ScatterDense range.
-  p.scale.assign(ntensors, -1.f);
+  p.range.assign(ntensors, -1.f);
   std::vector<int> state(ntensors, 0);
   std::function<float(int)> req = [&](int t) -> float {
-    if (state[t]) return p.scale[t];
+    if (state[t]) return p.range[t];
     state[t] = 1;
     float res = -1.f;
     for (auto& c : p.consumers[t]) {
       const NodeDesc& n = nodes[c.first];
       if (n.op == Op::Conv && p.comp[c.first] == SCN_PRECISION_INT8) {
-        res = n.in_range / 127.f;
+        res = n.in_range;
         break;
       }
     }
@@ -258,7 +258,7 @@ static Plan make_plan(const std::vector<NodeDesc>& nodes, size_t ntensors, int e
       for (auto& c : p.consumers[t]) {
         const NodeDesc& n = nodes[c.first];
         if (n.op == Op::Add && p.comp[c.first] == SCN_PRECISION_INT8) {
-          res = (c.second == 0 ? n.a_range : n.b_range) / 127.f;
+          res = c.second == 0 ? n.a_range : n.b_range;
           break;
         }
       }
@@ -266,11 +266,11 @@ static Plan make_plan(const std::vector<NodeDesc>& nodes, size_t ntensors, int e
       for (auto& c : p.consumers[t]) {
         const NodeDesc& n = nodes[c.first];
         if (n.op == Op::Dense && n.dense_range > 0.f) {
-          res = n.dense_range / 127.f;
+          res = n.dense_range;
           break;
         }
       }
-    p.scale[t] = res;
+    p.range[t] = res;
     return res;
   };
   for (size_t t = 0; t < ntensors; ++t) req((int)t);
@@ -418,14 +418,14 @@ static bool build_engine(scn_engine& e) {
         st.coord_out = slot.coord_out;
         st.t_in = n.in[0];
         const int want_dtype = comp == SCN_PRECISION_INT8 ? SCN_DTYPE_INT8 : SCN_DTYPE_FP16;
-        float want_scale = 1.f;
+        float want_range = 0.f;
         bool need_convert = false;
         if (comp == SCN_PRECISION_INT8) {
           if (x.dtype == SCN_DTYPE_INT8) {
-            st.x_scale = x.scale;
+            st.x_range = x.range;
           } else {
-            want_scale = n.in_range / 127.f;
-            st.x_scale = want_scale;
+            want_range = n.in_range;
+            st.x_range = want_range;
             need_convert = true;
           }
         } else if (x.dtype == SCN_DTYPE_INT8) {
@@ -436,14 +436,14 @@ static bool build_engine(scn_engine& e) {
         st.t_conv_in = n.in[0];
         if (need_convert) {
           char keybuf[128];
-          snprintf(keybuf, sizeof(keybuf), "%d:%d:%a:%u", n.in[0], want_dtype, (double)want_scale, w->cin_pad);
+          snprintf(keybuf, sizeof(keybuf), "%d:%d:%a:%u", n.in[0], want_dtype, (double)want_range, w->cin_pad);
           auto it = conversions.find(keybuf);
           if (it == conversions.end()) {
             e.tensors.emplace_back();
             RtTensor& cv = e.tensors.back();
             RtTensor& xx = e.tensors[n.in[0]];  // (re-take: the vector may have grown)
             cv.dtype = want_dtype;
-            cv.scale = want_scale;
+            cv.range = want_range;
             cv.c = xx.c;
             cv.ld = w->cin_pad;
             cv.coord = xx.coord;
@@ -469,8 +469,8 @@ static bool build_engine(scn_engine& e) {
         st.relu = n.activation == "ReLU" ? 1 : 0;
         if (!n.activation.empty() && n.activation != "ReLU" && n.activation != "None")
           SCN_LOGW("node %s: activation '%s' is not supported and is ignored", n.name.c_str(), n.activation.c_str());
-        int out_dtype = (plan.outp[i] == SCN_PRECISION_INT8 && plan.scale[n.out] > 0.f) ? SCN_DTYPE_INT8 : SCN_DTYPE_FP16;
-        float out_scale = out_dtype == SCN_DTYPE_INT8 ? plan.scale[n.out] : 1.f;
+        int out_dtype = (plan.outp[i] == SCN_PRECISION_INT8 && plan.range[n.out] > 0.f) ? SCN_DTYPE_INT8 : SCN_DTYPE_FP16;
+        float out_range = out_dtype == SCN_DTYPE_INT8 ? plan.range[n.out] : 0.f;
         if (plan.outp[i] == SCN_PRECISION_INT8 && out_dtype != SCN_DTYPE_INT8)
           SCN_LOGW("node %s: int8 output requested but no consumer provides a dynamic range; using fp16", n.name.c_str());
         if (!keep_all) {
@@ -487,18 +487,18 @@ static bool build_engine(scn_engine& e) {
               st.fused_add = true;
               st.t_in2 = other;
               st.mid_dtype = out_dtype;
-              st.mid_scale = out_scale;
+              st.mid_range = out_range;
               const bool add_i8 = plan.comp[c1] == SCN_PRECISION_INT8;
-              const float rq_self = add_i8 ? (slot_a == 0 ? an.a_range : an.b_range) / 127.f : 0.f;
-              const float rq_other = add_i8 ? (slot_a == 0 ? an.b_range : an.a_range) / 127.f : 0.f;
+              const float rq_self = add_i8 ? (slot_a == 0 ? an.a_range : an.b_range) : 0.f;
+              const float rq_other = add_i8 ? (slot_a == 0 ? an.b_range : an.a_range) : 0.f;
               st.a_rq = (add_i8 && out_dtype == SCN_DTYPE_FP16) ? rq_self : 0.f;
               st.b_rq = (add_i8 && ot.dtype == SCN_DTYPE_FP16) ? rq_other : 0.f;
               fused_away[c1] = true;
               e.tensors[n.out].coord = slot.coord_out;
               e.tensors[n.out].c = cout;
               t_out = an.out;
-              out_dtype = (plan.outp[c1] == SCN_PRECISION_INT8 && plan.scale[an.out] > 0.f) ? SCN_DTYPE_INT8 : SCN_DTYPE_FP16;
-              out_scale = out_dtype == SCN_DTYPE_INT8 ? plan.scale[an.out] : 1.f;
+              out_dtype = (plan.outp[c1] == SCN_PRECISION_INT8 && plan.range[an.out] > 0.f) ? SCN_DTYPE_INT8 : SCN_DTYPE_FP16;
+              out_range = out_dtype == SCN_DTYPE_INT8 ? plan.range[an.out] : 0.f;
               int c2 = single_consumer(an.out);
               if (c2 >= 0 && nodes[c2].op == Op::Relu && c2 == c1 + 1) {
                 st.relu2 = 1;
@@ -520,7 +520,7 @@ static bool build_engine(scn_engine& e) {
         }
         RtTensor& o = e.tensors[t_out];
         o.dtype = out_dtype;
-        o.scale = out_scale;
+        o.range = out_range;
         o.c = cout;
         o.ld = (uint32_t)w->mtiles * 16;
         o.coord = slot.coord_out;
@@ -545,11 +545,11 @@ static bool build_engine(scn_engine& e) {
         st.t_in2 = n.in[1];
         st.coord = a.coord;
         const bool add_i8 = plan.comp[i] == SCN_PRECISION_INT8;
-        st.add_a_rq = (add_i8 && a.dtype == SCN_DTYPE_FP16) ? n.a_range / 127.f : 0.f;
-        st.add_b_rq = (add_i8 && b.dtype == SCN_DTYPE_FP16) ? n.b_range / 127.f : 0.f;
+        st.add_a_rq = (add_i8 && a.dtype == SCN_DTYPE_FP16) ? n.a_range : 0.f;
+        st.add_b_rq = (add_i8 && b.dtype == SCN_DTYPE_FP16) ? n.b_range : 0.f;
         int t_out = n.out;
-        const int out_dtype = (plan.outp[i] == SCN_PRECISION_INT8 && plan.scale[n.out] > 0.f) ? SCN_DTYPE_INT8 : SCN_DTYPE_FP16;
-        const float out_scale = out_dtype == SCN_DTYPE_INT8 ? plan.scale[n.out] : 1.f;
+        const int out_dtype = (plan.outp[i] == SCN_PRECISION_INT8 && plan.range[n.out] > 0.f) ? SCN_DTYPE_INT8 : SCN_DTYPE_FP16;
+        const float out_range = out_dtype == SCN_DTYPE_INT8 ? plan.range[n.out] : 0.f;
         if (!keep_all) {
           int c1 = single_consumer(n.out);
           if (c1 >= 0 && nodes[c1].op == Op::Relu && c1 == (int)i + 1) {
@@ -563,7 +563,7 @@ static bool build_engine(scn_engine& e) {
         }
         RtTensor& o = e.tensors[t_out];
         o.dtype = out_dtype;
-        o.scale = out_scale;
+        o.range = out_range;
         o.c = a.c;
         o.ld = a.ld;
         o.coord = a.coord;
@@ -587,7 +587,7 @@ static bool build_engine(scn_engine& e) {
         st.coord = x.coord;
         RtTensor& o = e.tensors[n.out];
         o.dtype = x.dtype;
-        o.scale = x.scale;
+        o.range = x.range;
         o.c = x.c;
         o.ld = x.ld;
         o.coord = x.coord;
@@ -744,6 +744,9 @@ static int allocate_runtime(scn_engine& e) {
       if (!s.rb.init(max_in, max_out, kvol)) return SCN_ERR_HIP;
       s.initialised = true;
     }
+    // everything a build would allocate lazily is allocated here: forward() must not allocate
+    int rc = s.subm ? s.rb.reserve_subm(false) : s.rb.reserve_sparse(e.coords[s.coord_out].grid, false);
+    if (rc) return rc;
   }
   const bool keep_all = (e.flags & SCN_BUILD_KEEP_ALL) != 0;
   for (size_t t = 0; t < e.tensors.size(); ++t) {
@@ -828,7 +831,7 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
       const RtTensor& x = e.tensors[st.t_in];
       RtTensor& o = e.tensors[st.t_out];
       const CoordSet& cs = e.coords[x.coord];
-      return convert_rows(x.data, x.dtype, (uint32_t)x.c, x.ld, x.scale, o.data, o.dtype, o.ld, o.ld, o.scale, 0,
+      return convert_rows(x.data, x.dtype, (uint32_t)x.c, x.ld, x.range, o.data, o.dtype, o.ld, o.ld, o.range, 0,
                           cs.n_bound, cs.n_dev, stream);
     }
     case StepKind::Conv: {
@@ -839,10 +842,10 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
       memset(&io, 0, sizeof(io));
       io.x_dev = x.data;
       io.x_ld = x.ld;
-      io.x_scale = st.x_scale;
+      io.x_dynamic_range = st.x_range;
       io.relu = st.relu;
       io.out_dtype = o.dtype;
-      io.out_scale = o.scale;
+      io.out_dynamic_range = o.range;
       io.out_dev = o.data;
       io.out_ld = o.ld;
       io.acc_dev = o.acc.p;
@@ -850,12 +853,12 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
         const RtTensor& r = e.tensors[st.t_in2];
         io.res_dev = r.data;
         io.res_dtype = r.dtype;
-        io.res_scale = r.scale;
+        io.res_dynamic_range = r.range;
         io.res_ld = r.ld;
         io.mid_dtype = st.mid_dtype;
-        io.mid_scale = st.mid_scale;
-        io.a_requant_scale = st.a_rq;
-        io.b_requant_scale = st.b_rq;
+        io.mid_dynamic_range = st.mid_range;
+        io.a_requant_range = st.a_rq;
+        io.b_requant_range = st.b_rq;
         io.relu_after_add = st.relu2;
       }
       return conv_forward(*e.convs[st.conv], s.rb.nbr.as<int32_t>(), s.rb.ld, s.rb.n_out_dev(), s.rb.n_bound_out, io,
@@ -866,25 +869,22 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
       const RtTensor& b = e.tensors[st.t_in2];
       RtTensor& o = e.tensors[st.t_out];
       const CoordSet& cs = e.coords[a.coord];
-      return add_relu(a.data, a.dtype, a.scale, st.add_a_rq, b.data, b.dtype, b.scale, st.add_b_rq, o.data, o.dtype,
-                      o.scale, st.relu, a.ld, cs.n_bound, cs.n_dev, stream);
+      return add_relu(a.data, a.dtype, a.range, st.add_a_rq, b.data, b.dtype, b.range, st.add_b_rq, o.data, o.dtype,
+                      o.range, st.relu, a.ld, cs.n_bound, cs.n_dev, stream);
     }
     case StepKind::Relu: {
       const RtTensor& x = e.tensors[st.t_in];
       RtTensor& o = e.tensors[st.t_out];
       const CoordSet& cs = e.coords[x.coord];
-      // value-preserving re-store with ReLU: int8 keeps its scale (q*s/s rounds back to q)
-      if (x.dtype == SCN_DTYPE_INT8)
-        return convert_rows(x.data, SCN_DTYPE_INT8, x.ld, x.ld, 1.f, o.data, SCN_DTYPE_INT8, o.ld, o.ld, 1.f, 1,
-                            cs.n_bound, cs.n_dev, stream);
-      return convert_rows(x.data, x.dtype, x.ld, x.ld, 1.f, o.data, o.dtype, o.ld, o.ld, 1.f, 1, cs.n_bound, cs.n_dev,
+      // value-preserving re-store with ReLU: a range of 127 makes the int8 <-> value mapping the identity
+      return convert_rows(x.data, x.dtype, x.ld, x.ld, 127.f, o.data, o.dtype, o.ld, o.ld, 127.f, 1, cs.n_bound, cs.n_dev,
                           stream);
     }
     case StepKind::Dense: {
       const RtTensor& x = e.tensors[st.t_in];
       RtTensor& o = e.tensors[st.t_out];
       const CoordSet& cs = e.coords[x.coord];
-      return scatter_dense(x.data, x.dtype, x.scale, (uint32_t)x.c, x.ld, cs.idx, cs.n_bound, cs.n_dev, st.dense_shape,
+      return scatter_dense(x.data, x.dtype, x.range, (uint32_t)x.c, x.ld, cs.idx, cs.n_bound, cs.n_dev, st.dense_shape,
                            st.has_perm ? st.perm : nullptr, o.data, stream);
     }
     case StepKind::Permute: {
@@ -1463,6 +1463,13 @@ int scn_engine_set_num_points_device_ptr(scn_engine* e, int index, const uint32_
   return SCN_OK;
 }
 
+int scn_engine_prepare(scn_engine* e, const int grid_size[3]) {
+  SCN_REQUIRE(e && grid_size, SCN_ERR_INVALID, "prepare: invalid arguments");
+  if (e->allocated && memcmp(e->alloc_grid, grid_size, 12) == 0) return SCN_OK;
+  memcpy(e->in_grid, grid_size, 12);
+  return allocate_runtime(*e);
+}
+
 int scn_engine_forward(scn_engine* e, void* stream_) {
   SCN_REQUIRE(e, SCN_ERR_INVALID, "forward: null engine");
   SCN_REQUIRE(e->input_set, SCN_ERR_INVALID, "forward: no input has been set");
@@ -1499,7 +1506,7 @@ static void fill_view(scn_engine* e, int t, scn_tensor_view* v) {
   v->name = (t < (int)e->tdesc.size()) ? e->tdesc[t].name.c_str() : "";
   v->features_dev = x.data;
   v->dtype = x.dtype;
-  v->scale = x.scale;
+  v->dynamic_range = x.range;
   if (x.dense) {
     v->ndim = (int)std::min<size_t>(x.shape.size(), 8);
     for (int j = 0; j < v->ndim; ++j) v->shape[j] = x.shape[j];

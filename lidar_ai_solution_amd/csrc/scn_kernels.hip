@@ -441,7 +441,8 @@ int Rulebook::build_subm(const int32_t* idx, uint32_t n, const uint32_t* n_dev, 
     hipLaunchKernelGGL(k_set_count, dim3(1), dim3(64), 0, stream, cnt, n_dev, n);
     SCN_HIP(hipGetLastError());
   } else {
-    if (own_in_table.cap < hash_capacity_for(max_in) && !own_in_table.alloc_for(max_in)) return SCN_ERR_HIP;
+    rc = reserve_subm(true);
+    if (rc) return rc;
     rc = hash_build(own_in_table, idx, n, n_dev, grid, cnt, stream);
     if (rc) return rc;
     in_table = &own_in_table;
@@ -450,6 +451,31 @@ int Rulebook::build_subm(const int32_t* idx, uint32_t n, const uint32_t* n_dev, 
   rc = launch_build_nbr(*this, idx, n, odd, stream);
   if (rc) return rc;
   built = true;
+  return SCN_OK;
+}
+
+// Allocates what a strided build needs for the given output grid (no-op when already large enough),
+// so that a later build only launches kernels.
+int Rulebook::reserve_sparse(const int out_grid[3], bool need_own_in_table) {
+  const size_t words = bitmap_words_for(out_grid);
+  if (words > bitmap_cap_words) {
+    if (!bitmap.alloc(words * 4)) return SCN_ERR_HIP;
+    if (!blocksum.alloc((words / kWordsPerBlock + 1) * 4)) return SCN_ERR_HIP;
+    if (!prefix.alloc(words * 4)) return SCN_ERR_HIP;
+    bitmap_cap_words = words;
+  }
+  bitmap_words = words;
+  if (out_idx.bytes < (size_t)std::max(max_out, 1u) * 16 && !out_idx.alloc((size_t)std::max(max_out, 1u) * 16))
+    return SCN_ERR_HIP;
+  if (out_table.cap < hash_capacity_for(max_out) && !out_table.alloc_for(max_out)) return SCN_ERR_HIP;
+  if (need_own_in_table && own_in_table.cap < hash_capacity_for(max_in) && !own_in_table.alloc_for(max_in))
+    return SCN_ERR_HIP;
+  return SCN_OK;
+}
+
+int Rulebook::reserve_subm(bool need_own_in_table) {
+  if (need_own_in_table && own_in_table.cap < hash_capacity_for(max_in) && !own_in_table.alloc_for(max_in))
+    return SCN_ERR_HIP;
   return SCN_OK;
 }
 
@@ -482,22 +508,15 @@ int Rulebook::build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev
     uint64_t b = std::min<uint64_t>((uint64_t)n * (uint64_t)geom.kvol, vol);
     n_bound_out = (uint32_t)std::min<uint64_t>(b, max_out);
   }
-  const size_t words = bitmap_words_for(geom.grid_out);
-  if (words != bitmap_words) {
-    if (!bitmap.alloc(words * 4)) return SCN_ERR_HIP;
-    if (!blocksum.alloc((words / kWordsPerBlock + 1) * 4)) return SCN_ERR_HIP;
-    if (!prefix.alloc(words * 4)) return SCN_ERR_HIP;
-    bitmap_words = words;
-  }
-  if (out_idx.bytes < (size_t)max_out * 16 && !out_idx.alloc((size_t)std::max(max_out, 1u) * 16)) return SCN_ERR_HIP;
-  if (out_table.cap < hash_capacity_for(max_out) && !out_table.alloc_for(max_out)) return SCN_ERR_HIP;
+  rc = reserve_sparse(geom.grid_out, shared_in_table == nullptr);
+  if (rc) return rc;
+  const size_t words = bitmap_words;
   out_indices = out_idx.as<int32_t>();
   uint32_t* cnt = counters.as<uint32_t>();
   // input table
   if (shared_in_table) {
     in_table = shared_in_table;
   } else {
-    if (own_in_table.cap < hash_capacity_for(max_in) && !own_in_table.alloc_for(max_in)) return SCN_ERR_HIP;
     rc = hash_build(own_in_table, idx, n, n_dev, grid, nullptr, stream);
     if (rc) return rc;
     in_table = &own_in_table;
@@ -628,26 +647,28 @@ struct ConvArgs {
   const float* wscale;
   const float* bias;
   int cout;
-  float x_scale;
+  float x_scale;            // amax_x / 127
   int relu;
   int out_dtype;
-  float out_scale;
+  float out_r;              // 127 / amax_out
   char* out;
   uint32_t out_ld;
   void* acc;
   const char* res;
   int res_dtype;
-  float res_scale;
+  float res_scale;          // amax_res / 127
   uint32_t res_ld;
   int mid_dtype;
-  float mid_scale;
-  float a_rq, b_rq;
+  float mid_s, mid_r;       // amax_mid / 127, 127 / amax_mid
+  float a_rq_s, a_rq_r;     // re-quantisation of an fp16 operand by an int8 Add (0 = none)
+  float b_rq_s, b_rq_r;
   int relu2;
   int debug;  // measurement knob: 1 = no gathers, 2 = no weight slab loads, 8 = no epilogue, 16 = no main loop
 };
 
-__device__ __forceinline__ float quant_f(float y, float s) {
-  float q = rintf(y / s);
+// int8 store of the fake-quant form: round(y * (127/amax)), saturated to +-127
+__device__ __forceinline__ float quant_f(float y, float r) {
+  float q = rintf(y * r);
   q = fminf(fmaxf(q, -127.f), 127.f);  // NaN -> -127 (fmaxf returns the non-NaN operand)
   return q;
 }
@@ -732,17 +753,17 @@ __device__ __forceinline__ void epilogue_store(const ConvArgs& a, uint32_t row, 
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         rv[j] = (float)r[j];
-        if (a.b_rq > 0.f) rv[j] = quant_f(rv[j], a.b_rq) * a.b_rq;
+        if (a.b_rq_r > 0.f) rv[j] = quant_f(rv[j], a.b_rq_r) * a.b_rq_s;
       }
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       float v;
       if (a.mid_dtype == SCN_DTYPE_INT8) {
-        v = quant_f(y[j], a.mid_scale) * a.mid_scale;
+        v = quant_f(y[j], a.mid_r) * a.mid_s;
       } else {
         v = half_round(y[j]);
-        if (a.a_rq > 0.f) v = quant_f(v, a.a_rq) * a.a_rq;
+        if (a.a_rq_r > 0.f) v = quant_f(v, a.a_rq_r) * a.a_rq_s;
       }
       v = v + rv[j];
       if (a.relu2) v = v > 0.f ? v : 0.f;
@@ -751,10 +772,10 @@ __device__ __forceinline__ void epilogue_store(const ConvArgs& a, uint32_t row, 
   }
   if (a.out_dtype == SCN_DTYPE_INT8) {
     char4 q;
-    q.x = (signed char)quant_f(y[0], a.out_scale);
-    q.y = (signed char)quant_f(y[1], a.out_scale);
-    q.z = (signed char)quant_f(y[2], a.out_scale);
-    q.w = (signed char)quant_f(y[3], a.out_scale);
+    q.x = (signed char)quant_f(y[0], a.out_r);
+    q.y = (signed char)quant_f(y[1], a.out_r);
+    q.z = (signed char)quant_f(y[2], a.out_r);
+    q.w = (signed char)quant_f(y[3], a.out_r);
     *reinterpret_cast<char4*>(a.out + (size_t)row * a.out_ld + co) = q;
   } else {
     typedef _Float16 v4h __attribute__((ext_vector_type(4)));
@@ -1062,7 +1083,7 @@ bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* 
           if (ci >= cin) break;
           const uint16_t hb = w_fp16[((size_t)co * kvol + k) * cin + ci];
           if (prec == SCN_PRECISION_INT8) {
-            float q = rintf(half_bits_to_float(hb) / ws[co]);
+            float q = rintf(half_bits_to_float(hb) * (127.f / ranges[co]));
             if (!(q >= -127.f)) q = -127.f;
             if (q > 127.f) q = 127.f;
             dst[e] = (uint8_t)(int8_t)q;
@@ -1167,22 +1188,31 @@ int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, cons
   a.wscale = w.wscale.as<float>();
   a.bias = w.bias.as<float>();
   a.cout = w.cout;
-  a.x_scale = io.x_scale;
+  auto s_of = [](float range) { return range > 0.f ? range / 127.f : 0.f; };
+  auto r_of = [](float range) { return range > 0.f ? 127.f / range : 0.f; };
+  a.x_scale = s_of(io.x_dynamic_range);
   a.relu = io.relu;
   a.out_dtype = io.out_dtype;
-  a.out_scale = io.out_scale;
+  a.out_r = r_of(io.out_dynamic_range);
   a.out = (char*)io.out_dev;
   a.out_ld = io.out_ld;
   a.acc = io.acc_dev;
   a.res = (const char*)io.res_dev;
   a.res_dtype = io.res_dtype;
-  a.res_scale = io.res_scale;
+  a.res_scale = s_of(io.res_dynamic_range);
   a.res_ld = io.res_ld;
   a.mid_dtype = io.mid_dtype;
-  a.mid_scale = io.mid_scale;
-  a.a_rq = io.a_requant_scale;
-  a.b_rq = io.b_requant_scale;
+  a.mid_s = s_of(io.mid_dynamic_range);
+  a.mid_r = r_of(io.mid_dynamic_range);
+  a.a_rq_s = s_of(io.a_requant_range);
+  a.a_rq_r = r_of(io.a_requant_range);
+  a.b_rq_s = s_of(io.b_requant_range);
+  a.b_rq_r = r_of(io.b_requant_range);
   a.relu2 = io.relu_after_add;
+  if (io.out_dtype == SCN_DTYPE_INT8)
+    SCN_REQUIRE(io.out_dynamic_range > 0.f, SCN_ERR_INVALID, "conv: int8 output needs out_dynamic_range > 0");
+  if (w.precision == SCN_PRECISION_INT8)
+    SCN_REQUIRE(io.x_dynamic_range > 0.f, SCN_ERR_INVALID, "conv: int8 input needs x_dynamic_range > 0");
   {
     static const int dbg = getenv("SCN_CONV_DEBUG") ? atoi(getenv("SCN_CONV_DEBUG")) : 0;
     a.debug = dbg;
@@ -1198,37 +1228,43 @@ int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, cons
 // --------------------------------------------------------------------------------------------
 // elementwise glue
 // --------------------------------------------------------------------------------------------
-__device__ __forceinline__ float load_value(const void* p, int dtype, size_t i, float scale, float rq) {
+// scale = amax/127 of an int8 operand; rq_s / rq_r = amax/127 and 127/amax of the re-quantisation an
+// int8 Add applies to an fp16 operand (0 = none)
+__device__ __forceinline__ float load_value(const void* p, int dtype, size_t i, float scale, float rq_s, float rq_r) {
   if (dtype == SCN_DTYPE_INT8) return (float)reinterpret_cast<const signed char*>(p)[i] * scale;
   float v = (float)reinterpret_cast<const _Float16*>(p)[i];
-  if (rq > 0.f) v = quant_f(v, rq) * rq;
+  if (rq_r > 0.f) v = quant_f(v, rq_r) * rq_s;
   return v;
 }
 
-__device__ __forceinline__ void store_value(void* p, int dtype, size_t i, float v, float scale) {
+// r = 127/amax of an int8 destination
+__device__ __forceinline__ void store_value(void* p, int dtype, size_t i, float v, float r) {
   if (dtype == SCN_DTYPE_INT8)
-    reinterpret_cast<signed char*>(p)[i] = (signed char)quant_f(v, scale);
+    reinterpret_cast<signed char*>(p)[i] = (signed char)quant_f(v, r);
   else
     reinterpret_cast<_Float16*>(p)[i] = (_Float16)v;
 }
 
 __global__ __launch_bounds__(256) void k_convert_rows(const void* in, int in_dtype, uint32_t in_c, uint32_t in_ld,
                                                       float in_scale, void* out, int out_dtype, uint32_t out_c,
-                                                      uint32_t out_ld, float out_scale, int relu, uint32_t n_bound,
+                                                      uint32_t out_ld, float out_r, int relu, uint32_t n_bound,
                                                       const uint32_t* n_dev) {
   const uint32_t n = eff_n(n_dev, n_bound);
   const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
   const uint32_t row = (uint32_t)(t / out_c), c = (uint32_t)(t % out_c);
   if (row >= n) return;
   float v = 0.f;
-  if (c < in_c) v = load_value(in, in_dtype, (size_t)row * in_ld + c, in_scale, 0.f);
+  if (c < in_c) v = load_value(in, in_dtype, (size_t)row * in_ld + c, in_scale, 0.f, 0.f);
   if (relu) v = v > 0.f ? v : 0.f;
-  store_value(out, out_dtype, (size_t)row * out_ld + c, v, out_scale);
+  store_value(out, out_dtype, (size_t)row * out_ld + c, v, out_r);
 }
 
-int convert_rows(const void* in, int in_dtype, uint32_t in_c, uint32_t in_ld, float in_scale, void* out,
-                 int out_dtype, uint32_t out_c, uint32_t out_ld, float out_scale, int relu, uint32_t n,
+// in_range / out_range: dynamic ranges (amax) of int8 operands; a range of 127 makes q <-> value the identity
+int convert_rows(const void* in, int in_dtype, uint32_t in_c, uint32_t in_ld, float in_range, void* out,
+                 int out_dtype, uint32_t out_c, uint32_t out_ld, float out_range, int relu, uint32_t n,
                  const uint32_t* n_dev, hipStream_t stream) {
+  const float in_scale = in_range > 0.f ? in_range / 127.f : 1.f;
+  const float out_scale = out_range > 0.f ? 127.f / out_range : 1.f;
   if (n == 0) return SCN_OK;
   SCN_REQUIRE(in && out && out_c > 0 && out_ld >= out_c && in_ld >= in_c, SCN_ERR_INVALID, "convert_rows: bad arguments");
   const size_t total = (size_t)n * out_c;
@@ -1238,26 +1274,35 @@ int convert_rows(const void* in, int in_dtype, uint32_t in_c, uint32_t in_ld, fl
   return SCN_OK;
 }
 
-__global__ __launch_bounds__(256) void k_add_relu(const void* a, int a_dtype, float a_scale, float a_rq, const void* b,
-                                                  int b_dtype, float b_scale, float b_rq, void* out, int out_dtype,
-                                                  float out_scale, int relu, uint32_t c, uint32_t n_bound,
-                                                  const uint32_t* n_dev) {
+struct AddOperand {
+  const void* p;
+  int dtype;
+  float scale, rq_s, rq_r;
+};
+
+__global__ __launch_bounds__(256) void k_add_relu(AddOperand a, AddOperand b, void* out, int out_dtype, float out_r,
+                                                  int relu, uint32_t c, uint32_t n_bound, const uint32_t* n_dev) {
   const size_t total = (size_t)eff_n(n_dev, n_bound) * c;
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= total) return;
-  float v = load_value(a, a_dtype, i, a_scale, a_rq) + load_value(b, b_dtype, i, b_scale, b_rq);
+  float v = load_value(a.p, a.dtype, i, a.scale, a.rq_s, a.rq_r) + load_value(b.p, b.dtype, i, b.scale, b.rq_s, b.rq_r);
   if (relu) v = v > 0.f ? v : 0.f;
-  store_value(out, out_dtype, i, v, out_scale);
+  store_value(out, out_dtype, i, v, out_r);
 }
 
-int add_relu(const void* a, int a_dtype, float a_scale, float a_rq, const void* b, int b_dtype, float b_scale,
-             float b_rq, void* out, int out_dtype, float out_scale, int relu, uint32_t c, uint32_t n,
+// *_range: dynamic range (amax) of an int8 operand; *_rq: range an int8 Add re-quantises an fp16 operand with
+int add_relu(const void* a, int a_dtype, float a_range, float a_rq, const void* b, int b_dtype, float b_range,
+             float b_rq, void* out, int out_dtype, float out_range, int relu, uint32_t c, uint32_t n,
              const uint32_t* n_dev, hipStream_t stream) {
   if (n == 0 || c == 0) return SCN_OK;
   SCN_REQUIRE(a && b && out, SCN_ERR_INVALID, "add_relu: null pointer");
   const size_t total = (size_t)n * c;
-  hipLaunchKernelGGL(k_add_relu, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, a_dtype, a_scale, a_rq,
-                     b, b_dtype, b_scale, b_rq, out, out_dtype, out_scale, relu, c, n, n_dev);
+  auto s_of = [](float r) { return r > 0.f ? r / 127.f : 0.f; };
+  auto r_of = [](float r) { return r > 0.f ? 127.f / r : 0.f; };
+  const AddOperand oa{a, a_dtype, s_of(a_range), s_of(a_rq), r_of(a_rq)};
+  const AddOperand ob{b, b_dtype, s_of(b_range), s_of(b_rq), r_of(b_rq)};
+  hipLaunchKernelGGL(k_add_relu, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, oa, ob, out, out_dtype,
+                     r_of(out_range), relu, c, n, n_dev);
   SCN_HIP(hipGetLastError());
   return SCN_OK;
 }
@@ -1279,13 +1324,14 @@ __global__ __launch_bounds__(256) void k_scatter_dense(const void* feat, int dty
   const uint32_t c = blockIdx.y;
   const int4 p = coords[row];
   if (p.x != 0 || p.y < 0 || p.y >= st.d0 || p.z < 0 || p.z >= st.d1 || p.w < 0 || p.w >= st.d2) return;
-  const float v = load_value(feat, dtype, (size_t)row * ld + c, scale, 0.f);
+  const float v = load_value(feat, dtype, (size_t)row * ld + c, scale, 0.f, 0.f);
   out[c * st.sc + p.y * st.s0 + p.z * st.s1 + p.w * st.s2] = (_Float16)v;
 }
 
-int scatter_dense(const void* feat, int dtype, float scale, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
+int scatter_dense(const void* feat, int dtype, float range, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
                   const uint32_t* n_dev, const int dense_shape[5], const int perm[5], void* out, hipStream_t stream) {
   SCN_REQUIRE(out && dense_shape, SCN_ERR_INVALID, "scatter_dense: null pointer");
+  const float scale = range > 0.f ? range / 127.f : 1.f;
   SCN_REQUIRE(dense_shape[0] == 1 && (uint32_t)dense_shape[1] == c, SCN_ERR_INVALID,
               "scatter_dense: output_shape must be [1, C=%u, D0, D1, D2]", c);
   int p[5] = {0, 1, 2, 3, 4};
@@ -1677,22 +1723,22 @@ int scn_conv_forward(const scn_conv* c, const scn_rulebook* rb, const scn_conv_i
 }
 
 // ---- elementwise / dense --------------------------------------------------------------------
-int scn_convert_rows(const void* in_dev, int in_dtype, uint32_t in_c, uint32_t in_ld, float in_scale, void* out_dev,
-                     int out_dtype, uint32_t out_c, uint32_t out_ld, float out_scale, int relu, uint32_t n,
+int scn_convert_rows(const void* in_dev, int in_dtype, uint32_t in_c, uint32_t in_ld, float in_range, void* out_dev,
+                     int out_dtype, uint32_t out_c, uint32_t out_ld, float out_range, int relu, uint32_t n,
                      const uint32_t* n_dev, void* stream) {
-  return convert_rows(in_dev, in_dtype, in_c, in_ld, in_scale, out_dev, out_dtype, out_c, out_ld, out_scale, relu, n,
+  return convert_rows(in_dev, in_dtype, in_c, in_ld, in_range, out_dev, out_dtype, out_c, out_ld, out_range, relu, n,
                       n_dev, (hipStream_t)stream);
 }
-int scn_add_relu(const void* a_dev, int a_dtype, float a_scale, float a_requant_scale, const void* b_dev, int b_dtype,
-                 float b_scale, float b_requant_scale, void* out_dev, int out_dtype, float out_scale, int relu,
+int scn_add_relu(const void* a_dev, int a_dtype, float a_range, float a_requant_range, const void* b_dev, int b_dtype,
+                 float b_range, float b_requant_range, void* out_dev, int out_dtype, float out_range, int relu,
                  uint32_t c, uint32_t n, const uint32_t* n_dev, void* stream) {
-  return add_relu(a_dev, a_dtype, a_scale, a_requant_scale, b_dev, b_dtype, b_scale, b_requant_scale, out_dev,
-                  out_dtype, out_scale, relu, c, n, n_dev, (hipStream_t)stream);
+  return add_relu(a_dev, a_dtype, a_range, a_requant_range, b_dev, b_dtype, b_range, b_requant_range, out_dev,
+                  out_dtype, out_range, relu, c, n, n_dev, (hipStream_t)stream);
 }
-int scn_scatter_dense(const void* feat_dev, int dtype, float scale, uint32_t c, uint32_t ld, const int32_t* indices_dev,
-                      uint32_t n, const uint32_t* n_dev, const int dense_shape[5], const int perm[5],
-                      void* out_fp16_dev, void* stream) {
-  return scatter_dense(feat_dev, dtype, scale, c, ld, indices_dev, n, n_dev, dense_shape, perm, out_fp16_dev,
+int scn_scatter_dense(const void* feat_dev, int dtype, float dynamic_range, uint32_t c, uint32_t ld,
+                      const int32_t* indices_dev, uint32_t n, const uint32_t* n_dev, const int dense_shape[5],
+                      const int perm[5], void* out_fp16_dev, void* stream) {
+  return scatter_dense(feat_dev, dtype, dynamic_range, c, ld, indices_dev, n, n_dev, dense_shape, perm, out_fp16_dev,
                        (hipStream_t)stream);
 }
 

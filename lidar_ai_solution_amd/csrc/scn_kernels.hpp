@@ -42,7 +42,7 @@ struct Rulebook {
   DevBuf out_idx;             // int32 [max_out][4] (strided)
   DevBuf counters;            // uint32: [0] n_out kept, [1] n_out before truncation, [2..] scratch
   DevBuf bitmap, blocksum, prefix;  // strided: occupancy bitmap of the output grid, per-block popcounts, per-word ranks
-  size_t bitmap_words = 0;
+  size_t bitmap_words = 0, bitmap_cap_words = 0;
   DevBuf pair_scratch;        // pair compaction: per (k, block) counts
   const int32_t* in_indices = nullptr;
   const int32_t* out_indices = nullptr;  // subm: aliases in_indices
@@ -50,6 +50,8 @@ struct Rulebook {
   bool built = false;
 
   bool init(uint32_t max_in_, uint32_t max_out_, int kvol);
+  int reserve_sparse(const int out_grid[3], bool need_own_in_table);
+  int reserve_subm(bool need_own_in_table);
   int build_subm(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3], const int ks[3],
                  const int dil[3], const CoordTable* shared_in_table, hipStream_t stream);
   int build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3], const int ks[3],
@@ -83,13 +85,14 @@ int hash_build(const CoordTable& t, const int32_t* idx, uint32_t n, const uint32
 int hash_query(const CoordTable& t, const int32_t* coords, uint32_t n, const int grid[3], int32_t* rows,
                hipStream_t stream);
 
-int convert_rows(const void* in, int in_dtype, uint32_t in_c, uint32_t in_ld, float in_scale, void* out,
-                 int out_dtype, uint32_t out_c, uint32_t out_ld, float out_scale, int relu, uint32_t n,
+// the float arguments below are dynamic ranges (amax) of int8 operands, see scn_c_api.h
+int convert_rows(const void* in, int in_dtype, uint32_t in_c, uint32_t in_ld, float in_range, void* out,
+                 int out_dtype, uint32_t out_c, uint32_t out_ld, float out_range, int relu, uint32_t n,
                  const uint32_t* n_dev, hipStream_t stream);
-int add_relu(const void* a, int a_dtype, float a_scale, float a_rq, const void* b, int b_dtype, float b_scale,
-             float b_rq, void* out, int out_dtype, float out_scale, int relu, uint32_t c, uint32_t n,
+int add_relu(const void* a, int a_dtype, float a_range, float a_rq, const void* b, int b_dtype, float b_range,
+             float b_rq, void* out, int out_dtype, float out_range, int relu, uint32_t c, uint32_t n,
              const uint32_t* n_dev, hipStream_t stream);
-int scatter_dense(const void* feat, int dtype, float scale, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
+int scatter_dense(const void* feat, int dtype, float range, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
                   const uint32_t* n_dev, const int dense_shape[5], const int perm[5], void* out, hipStream_t stream);
 
 int permute_dense(const void* in, const int64_t in_shape[5], const int perm[5], void* out, hipStream_t stream);

@@ -50,7 +50,8 @@ class TensorView:
         self.indices_ptr = v.indices_dev
         self.num_ptr = v.num_dev
         self.grid_size = [int(x) for x in v.grid_size]
-        self.scale = float(v.scale)
+        self.dynamic_range = float(v.dynamic_range)  # int8 tensors: amax; value = q * (amax / 127)
+        self.scale = float(np.float32(v.dynamic_range) / np.float32(127.0))
         self.dense = v.indices_dev is None
 
     def _copy(self, ptr, shape, tdtype):

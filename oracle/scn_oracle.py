@@ -13,11 +13,13 @@ Precision rules stated by this build (the closed engine's are not recoverable):
     `precision` attribute is "int8" and it has an input range and per-channel weight ranges;
     an Add computes in int8 when `precision` is "int8" and both input ranges are set.
   * a tensor is stored int8 when its producer's `output_precision` is "int8" and some consumer
-    fixes its scale: an int8 conv's `input_dynamic_range` first, else (through Relu) the next
-    consumer, else an int8 Add's `inputK_dynamic_range`.  scale = range / 127 in fp32.
-  * int8 conv: Wq = clamp(rint(W / s_w[c])), acc int32, y = acc * (s_x * s_w[c]) + bias (two fp32
-    roundings), ReLU, then int8 store clamp(rint(y / s_out), +-127) or fp16 store.
-  * Add: value of an int8 operand is q * scale(tensor); one fp32 add; same stores.
+    fixes its dynamic range (amax): an int8 conv's `input_dynamic_range` first, else (through Relu)
+    the next consumer, else an int8 Add's `inputK_dynamic_range`.
+  * quantisation follows pytorch-quantization's fake-quant: q = clamp(rint(x * (127/amax)), +-127);
+    the value of an int8 element is q * (amax/127); both factors are computed in fp32.
+  * int8 conv: Wq from the per-channel weight ranges the same way, acc int32,
+    y = acc * (s_x * s_w[c]) + bias (two fp32 roundings), ReLU, then int8 or fp16 store.
+  * Add: value of an int8 operand is q * (amax(tensor)/127); one fp32 add; same stores.
 """
 from __future__ import annotations
 
@@ -161,8 +163,9 @@ def quantize_weights(w_f16: np.ndarray, ranges) -> Tuple[np.ndarray, np.ndarray]
     """[Cout,K0,K1,K2,Cin] fp16 -> ([kvol][cout][cin] int8, s_w[cout] fp32)."""
     cout, cin = w_f16.shape[0], w_f16.shape[-1]
     s_w = (np.asarray(ranges, np.float32) / f32(127.0)).astype(np.float32)
+    r_w = (f32(127.0) / np.asarray(ranges, np.float32)).astype(np.float32)
     w = w_f16.astype(np.float32).reshape(cout, -1, cin)
-    q = np.rint(w / s_w[:, None, None])
+    q = np.rint(w * r_w[:, None, None])
     q = np.clip(q, -127, 127).astype(np.int8)
     return np.ascontiguousarray(q.transpose(1, 0, 2)), s_w
 
@@ -189,7 +192,7 @@ def conv_f32_acc(x_f32: np.ndarray, w_f32: np.ndarray, rb: Rulebook) -> np.ndarr
 
 
 def epilogue(acc: np.ndarray, scale: Optional[np.ndarray], bias_f32: np.ndarray, relu: bool, out_int8: bool,
-             s_out: float = 1.0) -> np.ndarray:
+             out_range: float = 127.0) -> np.ndarray:
     n, cout = acc.shape
     out = np.empty((n, cout), np.int8 if out_int8 else np.float16)
     oi8 = _p(out) if out_int8 else None
@@ -198,36 +201,43 @@ def epilogue(acc: np.ndarray, scale: Optional[np.ndarray], bias_f32: np.ndarray,
     if acc.dtype == np.int32:
         lib().scn_ref_epilogue_int32(_p(np.ascontiguousarray(acc)), C.c_int64(n), C.c_int(cout),
                                      _p(np.ascontiguousarray(scale, np.float32)), _p(bias), C.c_int(int(relu)),
-                                     C.c_float(s_out), oi8, of16)
+                                     C.c_float(out_range), oi8, of16)
     else:
         lib().scn_ref_epilogue_f32(_p(np.ascontiguousarray(acc, np.float32)), C.c_int64(n), C.c_int(cout), _p(bias),
-                                   C.c_int(int(relu)), C.c_float(s_out), oi8, of16)
+                                   C.c_int(int(relu)), C.c_float(out_range), oi8, of16)
     return out
 
 
-def quantize(x_f16: np.ndarray, scale: float) -> np.ndarray:
+def quantize(x_f16: np.ndarray, rng: float) -> np.ndarray:
     x = np.ascontiguousarray(x_f16, np.float16)
     q = np.empty(x.shape, np.int8)
-    lib().scn_ref_quantize(_p(x.view(np.uint16)), C.c_int64(x.size), C.c_float(scale), _p(q))
+    lib().scn_ref_quantize(_p(x.view(np.uint16)), C.c_int64(x.size), C.c_float(rng), _p(q))
     return q
 
 
-def dequantize(q_i8: np.ndarray, scale: float) -> np.ndarray:
+def quantize_f32(x_f32: np.ndarray, rng: float) -> np.ndarray:
+    x = np.ascontiguousarray(x_f32, np.float32)
+    q = np.empty(x.shape, np.int8)
+    lib().scn_ref_quantize_f32(_p(x), C.c_int64(x.size), C.c_float(rng), _p(q))
+    return q
+
+
+def dequantize(q_i8: np.ndarray, rng: float) -> np.ndarray:
     q = np.ascontiguousarray(q_i8, np.int8)
     x = np.empty(q.shape, np.float16)
-    lib().scn_ref_dequantize(_p(q), C.c_int64(q.size), C.c_float(scale), _p(x.view(np.uint16)))
+    lib().scn_ref_dequantize(_p(q), C.c_int64(q.size), C.c_float(rng), _p(x.view(np.uint16)))
     return x
 
 
-def add(a: np.ndarray, a_scale: float, b: np.ndarray, b_scale: float, relu: bool, out_int8: bool,
-        s_out: float = 1.0) -> np.ndarray:
+def add(a: np.ndarray, a_range: float, b: np.ndarray, b_range: float, relu: bool, out_int8: bool,
+        out_range: float = 127.0) -> np.ndarray:
     a = np.ascontiguousarray(a)
     b = np.ascontiguousarray(b)
     out = np.empty(a.shape, np.int8 if out_int8 else np.float16)
     lib().scn_ref_add(_p(a) if a.dtype == np.int8 else None, _p(a.view(np.uint16)) if a.dtype == np.float16 else None,
-                      C.c_float(a_scale), _p(b) if b.dtype == np.int8 else None,
-                      _p(b.view(np.uint16)) if b.dtype == np.float16 else None, C.c_float(b_scale),
-                      C.c_int64(a.size), C.c_int(int(relu)), C.c_float(s_out), _p(out) if out_int8 else None,
+                      C.c_float(a_range), _p(b) if b.dtype == np.int8 else None,
+                      _p(b.view(np.uint16)) if b.dtype == np.float16 else None, C.c_float(b_range),
+                      C.c_int64(a.size), C.c_int(int(relu)), C.c_float(out_range), _p(out) if out_int8 else None,
                       None if out_int8 else _p(out.view(np.uint16)))
     return out
 
@@ -243,8 +253,10 @@ def scatter_dense(feat: np.ndarray, indices: np.ndarray, dims) -> np.ndarray:
 
 # ------------------------------------------------------------------------------- graph walk
 class SparseT:
-    def __init__(self, feat, scale, indices, grid):
-        self.feat, self.scale, self.indices, self.grid = feat, scale, indices, list(grid)
+    """features (fp16, or int8 with its dynamic range `rng`), indices, grid."""
+
+    def __init__(self, feat, rng, indices, grid):
+        self.feat, self.rng, self.indices, self.grid = feat, rng, indices, list(grid)
 
 
 def _consumers(graph):
@@ -276,8 +288,8 @@ def node_precisions(graph, engine_precision: str):
     return out
 
 
-def tensor_scales(graph, prec):
-    """tensor name -> fp32 scale fixed by its consumers (None when no consumer fixes one)."""
+def tensor_ranges(graph, prec):
+    """tensor name -> dynamic range (amax) fixed by its consumers (None when no consumer fixes one)."""
     cons = _consumers(graph)
     memo: Dict[str, Optional[np.float32]] = {}
 
@@ -289,7 +301,7 @@ def tensor_scales(graph, prec):
         cl = cons.get(t, [])
         for n, _ in cl:
             if n.op_type == "SparseConvolution" and prec[n.name][0] == "int8":
-                res = f32(n.attrs["input_dynamic_range"]) / f32(127.0)
+                res = f32(n.attrs["input_dynamic_range"])
                 break
         if res is None:
             for n, _ in cl:
@@ -300,12 +312,12 @@ def tensor_scales(graph, prec):
         if res is None:
             for n, slot in cl:
                 if n.op_type in ("Add", "QuantAdd") and prec[n.name][0] == "int8":
-                    res = f32(n.attrs[f"input{slot}_dynamic_range"]) / f32(127.0)
+                    res = f32(n.attrs[f"input{slot}_dynamic_range"])
                     break
         if res is None:
             for n, _ in cl:
                 if n.op_type == "ScatterDense" and float(n.attrs.get("input_dynamic_range", 0.0)) > 0:
-                    res = f32(n.attrs["input_dynamic_range"]) / f32(127.0)
+                    res = f32(n.attrs["input_dynamic_range"])
                     break
         memo[t] = res
         return res
@@ -321,23 +333,23 @@ def run_graph(graph, features_f16: np.ndarray, indices: np.ndarray, grid, precis
     """Walks the graph.  Returns {output name: ndarray (dense) or SparseT}.
 
     record, when given, receives per node name a dict with the rulebook, the accumulators (`acc`)
-    and the stored output (`out`, plus `scale` for int8) of that node.
+    and the stored output (`out`, plus its dynamic `range` for int8) of that node.
     override maps a tensor name to stored features that replace what the walk computed for that
     tensor (same dtype and shape).  Tests use it to re-base the walk on the device's own output of
     an fp16-computed node, whose summation order the oracle does not model, so that every int8 node
     downstream sees identical inputs and can be compared bit for bit.
     """
     prec = node_precisions(graph, precision)
-    scales = tensor_scales(graph, prec)
+    ranges = tensor_ranges(graph, prec)
     T: Dict[str, object] = {graph.inputs[0]: SparseT(np.ascontiguousarray(features_f16, np.float16), None,
                                                      np.ascontiguousarray(indices, np.int32), grid)}
     rb_cache: Dict[str, Rulebook] = {}
 
     def stored(out_prec, name):
-        """(store int8?, scale) for an output tensor."""
-        if out_prec == "int8" and scales.get(name) is not None:
-            return True, float(scales[name])
-        return False, 1.0
+        """(store int8?, dynamic range) for an output tensor."""
+        if out_prec == "int8" and ranges.get(name) is not None:
+            return True, float(ranges[name])
+        return False, 127.0
 
     for n in graph.nodes:
         comp, outp = prec[n.name]
@@ -365,50 +377,51 @@ def run_graph(graph, features_f16: np.ndarray, indices: np.ndarray, grid, precis
                     if key:
                         rb_cache[ck] = rb
             relu = a.get("activation", "") == "ReLU"
-            o_i8, s_out = stored(outp, n.outputs[0])
+            o_i8, r_out = stored(outp, n.outputs[0])
             if comp == "int8":
                 if x.feat.dtype == np.int8:
-                    xq, s_x = x.feat, f32(x.scale)
+                    xq, x_rng = x.feat, f32(x.rng)
                 else:
-                    s_x = f32(a["input_dynamic_range"]) / f32(127.0)
-                    xq = quantize(x.feat, float(s_x))
+                    x_rng = f32(a["input_dynamic_range"])
+                    xq = quantize(x.feat, float(x_rng))
+                s_x = x_rng / f32(127.0)
                 wq, s_w = quantize_weights(w, a["weight_dynamic_ranges"])
                 acc = conv_int8_acc(xq, wq, rb)
-                out = epilogue(acc, (s_x * s_w).astype(np.float32), bias, relu, o_i8, s_out)
+                out = epilogue(acc, (s_x * s_w).astype(np.float32), bias, relu, o_i8, r_out)
             else:
-                xf = x.feat if x.feat.dtype == np.float16 else dequantize(x.feat, float(x.scale))
+                xf = x.feat if x.feat.dtype == np.float16 else dequantize(x.feat, float(x.rng))
                 cout, cin = w.shape[0], w.shape[-1]
                 wf = np.ascontiguousarray(w.astype(np.float32).reshape(cout, -1, cin).transpose(1, 0, 2))
                 acc = conv_f32_acc(xf.astype(np.float32), wf, rb)
-                out = epilogue(acc, None, bias, relu, o_i8, s_out)
-            T[n.outputs[0]] = SparseT(out, s_out if o_i8 else None, rb.out_indices, rb.out_grid)
+                out = epilogue(acc, None, bias, relu, o_i8, r_out)
+            T[n.outputs[0]] = SparseT(out, r_out if o_i8 else None, rb.out_indices, rb.out_grid)
             if rec is not None:
-                rec.update(rulebook=rb, acc=acc, out=out, scale=s_out if o_i8 else None)
+                rec.update(rulebook=rb, acc=acc, out=out, range=r_out if o_i8 else None)
         elif n.op_type in ("Add", "QuantAdd"):
             A: SparseT = T[n.inputs[0]]
             B: SparseT = T[n.inputs[1]]
-            fa, sa, fb, sb = A.feat, A.scale, B.feat, B.scale
+            fa, ra, fb, rb_ = A.feat, A.rng, B.feat, B.rng
             if comp == "int8":
                 if fa.dtype == np.float16:
-                    sa = float(f32(n.attrs["input0_dynamic_range"]) / f32(127.0))
-                    fa = quantize(fa, sa)
+                    ra = float(f32(n.attrs["input0_dynamic_range"]))
+                    fa = quantize(fa, ra)
                 if fb.dtype == np.float16:
-                    sb = float(f32(n.attrs["input1_dynamic_range"]) / f32(127.0))
-                    fb = quantize(fb, sb)
-            o_i8, s_out = stored(outp, n.outputs[0])
-            out = add(fa, sa or 1.0, fb, sb or 1.0, False, o_i8, s_out)
-            T[n.outputs[0]] = SparseT(out, s_out if o_i8 else None, A.indices, A.grid)
+                    rb_ = float(f32(n.attrs["input1_dynamic_range"]))
+                    fb = quantize(fb, rb_)
+            o_i8, r_out = stored(outp, n.outputs[0])
+            out = add(fa, ra or 127.0, fb, rb_ or 127.0, False, o_i8, r_out)
+            T[n.outputs[0]] = SparseT(out, r_out if o_i8 else None, A.indices, A.grid)
             if rec is not None:
-                rec.update(out=out, scale=s_out if o_i8 else None)
+                rec.update(out=out, range=r_out if o_i8 else None)
         elif n.op_type == "Relu":
             X: SparseT = T[n.inputs[0]]
             out = np.maximum(X.feat, X.feat.dtype.type(0))
-            T[n.outputs[0]] = SparseT(out, X.scale, X.indices, X.grid)
+            T[n.outputs[0]] = SparseT(out, X.rng, X.indices, X.grid)
             if rec is not None:
-                rec.update(out=out, scale=X.scale)
+                rec.update(out=out, range=X.rng)
         elif n.op_type == "ScatterDense":
             X = T[n.inputs[0]]
-            feat = X.feat if X.feat.dtype == np.float16 else dequantize(X.feat, float(X.scale))
+            feat = X.feat if X.feat.dtype == np.float16 else dequantize(X.feat, float(X.rng))
             oshape = [int(v) for v in n.attrs["output_shape"]]
             dense = scatter_dense(feat, X.indices, oshape[2:5])
             T[n.outputs[0]] = dense

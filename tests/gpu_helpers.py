@@ -119,14 +119,14 @@ class GpuConv:
             self.L.scn_conv_destroy(self.h)
             self.h = None
 
-    def forward(self, rb, x_dev, n_out, x_scale=1.0, relu=False, out_int8=False, out_scale=1.0, want_acc=False, **res):
+    def forward(self, rb, x_dev, n_out, x_range=127.0, relu=False, out_int8=False, out_range=127.0, want_acc=False, **res):
         io = capi.ConvIO()
         io.x_dev = x_dev.data_ptr()
         io.x_ld = x_dev.shape[1]
-        io.x_scale = x_scale
+        io.x_dynamic_range = x_range
         io.relu = int(relu)
         io.out_dtype = capi.DTYPE_INT8 if out_int8 else capi.DTYPE_FP16
-        io.out_scale = out_scale
+        io.out_dynamic_range = out_range
         out = torch.zeros((max(n_out, 1), self.cout), dtype=torch.int8 if out_int8 else torch.float16, device=DEV)
         io.out_dev = out.data_ptr()
         io.out_ld = self.cout
@@ -138,12 +138,12 @@ class GpuConv:
             r = res["res"]
             io.res_dev = r.data_ptr()
             io.res_dtype = capi.DTYPE_INT8 if r.dtype == torch.int8 else capi.DTYPE_FP16
-            io.res_scale = res.get("res_scale", 1.0)
+            io.res_dynamic_range = res.get("res_range", 127.0)
             io.res_ld = r.shape[1]
             io.mid_dtype = capi.DTYPE_INT8 if res.get("mid_int8", False) else capi.DTYPE_FP16
-            io.mid_scale = res.get("mid_scale", 1.0)
-            io.a_requant_scale = res.get("a_rq", 0.0)
-            io.b_requant_scale = res.get("b_rq", 0.0)
+            io.mid_dynamic_range = res.get("mid_range", 127.0)
+            io.a_requant_range = res.get("a_rq", 0.0)
+            io.b_requant_range = res.get("b_rq", 0.0)
             io.relu_after_add = int(res.get("relu2", False))
         capi.check(self.L.scn_conv_forward(self.h, rb.h, C.byref(io), stream()))
         torch.cuda.synchronize()

@@ -152,18 +152,19 @@ def test_config1_single_int8_subm_layer():
     idx = synth.uniform_voxels(0, 20000, grid)
     x = rng.integers(-127, 128, (20000, 16)).astype(np.int8)
     w, b, ranges = _weights(rng, 16, (3, 3, 3), 16)
-    s_x = 0.05
+    x_range = np.float32(0.05 * 127)  # a per-tensor activation scale of 0.05
+    s_x = x_range / np.float32(127)
     ref_rb = O.rulebook_subm(idx, grid, (3, 3, 3))
     wq, s_w = O.quantize_weights(w, ranges)
     acc_ref = O.conv_int8_acc(x, wq, ref_rb)
-    scale = (np.float32(s_x) * s_w).astype(np.float32)
+    scale = (s_x * s_w).astype(np.float32)
     y = np.maximum(acc_ref.astype(np.float32) * scale + b.astype(np.float32), 0)
-    s_out = float(np.float32(np.percentile(y, 99.99)) / np.float32(127))
-    out_ref = O.epilogue(acc_ref, scale, b.astype(np.float32), True, True, s_out)
+    out_range = float(np.float32(np.percentile(y, 99.99)))  # output range fixed up front: 99.99th percentile
+    out_ref = O.epilogue(acc_ref, scale, b.astype(np.float32), True, True, out_range)
     rb = GpuRulebook(20000, 20000, 27)
     rb.build_subm(to_dev(idx), 20000, grid, (3, 3, 3))
     conv = GpuConv(w, ranges, b, capi.PRECISION_INT8)
-    out, acc = conv.forward(rb, to_dev(x), 20000, x_scale=s_x, relu=True, out_int8=True, out_scale=s_out, want_acc=True)
+    out, acc = conv.forward(rb, to_dev(x), 20000, x_range=float(x_range), relu=True, out_int8=True, out_range=out_range, want_acc=True)
     assert np.array_equal(acc.cpu().numpy(), acc_ref)
     assert np.array_equal(out.cpu().numpy(), out_ref)
     assert ref_rb.num_pairs >= 20000 and np.abs(out_ref).max() > 20
@@ -183,7 +184,8 @@ def test_int8_conv_shapes_bit_exact(cin, cout, centerpoint_input):
     note(f"int8 conv {cin}->{cout} {'subm' if subm else 'strided'} on {n} fixture voxels")
     x = rng.integers(-127, 128, (n, cin)).astype(np.int8)
     w, b, ranges = _weights(rng, cout, (3, 3, 3), cin)
-    s_x, s_out = 0.031, 0.043
+    x_range, out_range = 3.9, 5.5
+    s_x = np.float32(x_range) / np.float32(127)
     if subm:
         ref_rb = O.rulebook_subm(idx, grid, (3, 3, 3))
         rb = GpuRulebook(n, n, 27)
@@ -194,12 +196,12 @@ def test_int8_conv_shapes_bit_exact(cin, cout, centerpoint_input):
         rb.build_sparse(to_dev(idx), n, grid, (3, 3, 3), (2, 2, 2), (1, 1, 1))
     wq, s_w = O.quantize_weights(w, ranges)
     acc_ref = O.conv_int8_acc(x, wq, ref_rb)
-    scale = (np.float32(s_x) * s_w).astype(np.float32)
+    scale = (s_x * s_w).astype(np.float32)
     conv = GpuConv(w, ranges, b, capi.PRECISION_INT8)
-    out, acc = conv.forward(rb, to_dev(x), ref_rb.n_out, x_scale=s_x, relu=True, out_int8=True, out_scale=s_out, want_acc=True)
+    out, acc = conv.forward(rb, to_dev(x), ref_rb.n_out, x_range=x_range, relu=True, out_int8=True, out_range=out_range, want_acc=True)
     assert np.array_equal(acc.cpu().numpy(), acc_ref)
-    assert np.array_equal(out.cpu().numpy(), O.epilogue(acc_ref, scale, b.astype(np.float32), True, True, s_out))
-    out16, _ = conv.forward(rb, to_dev(x), ref_rb.n_out, x_scale=s_x, relu=False, out_int8=False)
+    assert np.array_equal(out.cpu().numpy(), O.epilogue(acc_ref, scale, b.astype(np.float32), True, True, out_range))
+    out16, _ = conv.forward(rb, to_dev(x), ref_rb.n_out, x_range=x_range, relu=False, out_int8=False)
     ref16 = O.epilogue(acc_ref, scale, b.astype(np.float32), False, False)
     assert np.array_equal(out16.cpu().numpy().view(np.uint16), ref16.view(np.uint16))
 
@@ -248,31 +250,31 @@ def test_fused_residual_epilogue_matches_unfused_oracle(centerpoint_input):
     x = rng.integers(-127, 128, (n, cin)).astype(np.int8)
     ident = rng.integers(0, 128, (n, cout)).astype(np.int8)
     w, b, ranges = _weights(rng, cout, (3, 3, 3), cin)
-    s_x, s_mid, s_res, s_out = 0.02, 0.035, 0.027, 0.05
+    x_range, mid_range, res_range, out_range = 2.5, 4.4, 3.4, 6.3
     ref_rb = O.rulebook_subm(idx, grid, (3, 3, 3))
     wq, s_w = O.quantize_weights(w, ranges)
     acc_ref = O.conv_int8_acc(x, wq, ref_rb)
-    scale = (np.float32(s_x) * s_w).astype(np.float32)
+    scale = ((np.float32(x_range) / np.float32(127)) * s_w).astype(np.float32)
     rb = GpuRulebook(n, n, 27)
     rb.build_subm(to_dev(idx), n, grid, (3, 3, 3))
     conv = GpuConv(w, ranges, b, capi.PRECISION_INT8)
     note("int8 conv -> int8 add -> relu")
-    mid = O.epilogue(acc_ref, scale, b.astype(np.float32), False, True, s_mid)
-    want = O.add(mid, s_mid, ident, s_res, True, True, s_out)
-    out, _ = conv.forward(rb, to_dev(x), n, x_scale=s_x, relu=False, out_int8=True, out_scale=s_out,
-                          res=to_dev(ident), res_scale=s_res, mid_int8=True, mid_scale=s_mid, relu2=True)
+    mid = O.epilogue(acc_ref, scale, b.astype(np.float32), False, True, mid_range)
+    want = O.add(mid, mid_range, ident, res_range, True, True, out_range)
+    out, _ = conv.forward(rb, to_dev(x), n, x_range=x_range, relu=False, out_int8=True, out_range=out_range,
+                          res=to_dev(ident), res_range=res_range, mid_int8=True, mid_range=mid_range, relu2=True)
     assert np.array_equal(out.cpu().numpy(), want)
     note("fp16-stored conv output and fp16 identity, int8 add re-quantising both, int8 out")
     ident16 = (rng.standard_normal((n, cout)) * 2).astype(np.float16)
     mid16 = O.epilogue(acc_ref, scale, b.astype(np.float32), False, False)
-    s_add = 0.04
-    want2 = O.add(O.quantize(mid16, s_add), s_add, O.quantize(ident16, s_add), s_add, True, True, s_out)
-    out2, _ = conv.forward(rb, to_dev(x), n, x_scale=s_x, relu=False, out_int8=True, out_scale=s_out,
-                           res=to_dev(ident16), mid_int8=False, a_rq=s_add, b_rq=s_add, relu2=True)
+    add_range = 5.1
+    want2 = O.add(O.quantize(mid16, add_range), add_range, O.quantize(ident16, add_range), add_range, True, True, out_range)
+    out2, _ = conv.forward(rb, to_dev(x), n, x_range=x_range, relu=False, out_int8=True, out_range=out_range,
+                           res=to_dev(ident16), mid_int8=False, a_rq=add_range, b_rq=add_range, relu2=True)
     assert np.array_equal(out2.cpu().numpy(), want2)
     note("fp16 add of fp16 operands, fp16 out")
-    want3 = O.add(mid16, 1.0, ident16, 1.0, True, False)
-    out3, _ = conv.forward(rb, to_dev(x), n, x_scale=s_x, relu=False, out_int8=False,
+    want3 = O.add(mid16, 127.0, ident16, 127.0, True, False)
+    out3, _ = conv.forward(rb, to_dev(x), n, x_range=x_range, relu=False, out_int8=False,
                            res=to_dev(ident16), mid_int8=False, relu2=True)
     assert np.array_equal(out3.cpu().numpy().view(np.uint16), want3.view(np.uint16))
 
@@ -284,10 +286,10 @@ def test_convert_add_and_dense():
     n, c = 5000, 32
     note("quantise / dequantise / pad rows")
     x = (rng.standard_normal((n, 5)) * 20).astype(np.float16)
-    s = 0.3
+    s = 38.1  # dynamic range
     out = torch.zeros((n, 16), dtype=torch.int8, device=DEV)
     d_x = to_dev(x)
-    capi.check(L.scn_convert_rows(ptr(d_x), capi.DTYPE_FP16, 5, 5, 1.0, ptr(out), capi.DTYPE_INT8, 16, 16, s, 0, n, None, stream()))
+    capi.check(L.scn_convert_rows(ptr(d_x), capi.DTYPE_FP16, 5, 5, 0.0, ptr(out), capi.DTYPE_INT8, 16, 16, s, 0, n, None, stream()))
     torch.cuda.synchronize()
     want = np.zeros((n, 16), np.int8)
     want[:, :5] = O.quantize(x, s)
@@ -295,11 +297,11 @@ def test_convert_add_and_dense():
     q = rng.integers(-127, 128, (n, c)).astype(np.int8)
     out = torch.zeros((n, c), dtype=torch.float16, device=DEV)
     d_q = to_dev(q)
-    capi.check(L.scn_convert_rows(ptr(d_q), capi.DTYPE_INT8, c, c, s, ptr(out), capi.DTYPE_FP16, c, c, 1.0, 0, n, None, stream()))
+    capi.check(L.scn_convert_rows(ptr(d_q), capi.DTYPE_INT8, c, c, s, ptr(out), capi.DTYPE_FP16, c, c, 0.0, 0, n, None, stream()))
     torch.cuda.synchronize()
     assert np.array_equal(out.cpu().numpy().view(np.uint16), O.dequantize(q, s).view(np.uint16))
     padded = torch.full((n, 8), 7, dtype=torch.float16, device=DEV)
-    capi.check(L.scn_convert_rows(ptr(d_x), capi.DTYPE_FP16, 5, 5, 1.0, ptr(padded), capi.DTYPE_FP16, 8, 8, 1.0, 0, n, None, stream()))
+    capi.check(L.scn_convert_rows(ptr(d_x), capi.DTYPE_FP16, 5, 5, 0.0, ptr(padded), capi.DTYPE_FP16, 8, 8, 0.0, 0, n, None, stream()))
     torch.cuda.synchronize()
     pw = np.zeros((n, 8), np.float16); pw[:, :5] = x
     assert np.array_equal(padded.cpu().numpy().view(np.uint16), pw.view(np.uint16))
@@ -309,18 +311,18 @@ def test_convert_add_and_dense():
     n_dev = torch.tensor([4321], dtype=torch.int32, device=DEV)
     out = torch.zeros((n, c), dtype=torch.int8, device=DEV)
     da, db = to_dev(a), to_dev(b)  # keep both alive: the caching allocator would hand b the memory of a
-    capi.check(L.scn_add_relu(ptr(da), capi.DTYPE_INT8, 0.03, 0.0, ptr(db), capi.DTYPE_INT8, 0.02, 0.0, ptr(out),
-                              capi.DTYPE_INT8, 0.04, 1, c, n, ptr(n_dev), stream()))
+    capi.check(L.scn_add_relu(ptr(da), capi.DTYPE_INT8, 3.8, 0.0, ptr(db), capi.DTYPE_INT8, 2.5, 0.0, ptr(out),
+                              capi.DTYPE_INT8, 5.1, 1, c, n, ptr(n_dev), stream()))
     torch.cuda.synchronize()
     got = out.cpu().numpy()
-    assert np.array_equal(got[:4321], O.add(a[:4321], 0.03, b[:4321], 0.02, True, True, 0.04)) and not got[4321:].any()
+    assert np.array_equal(got[:4321], O.add(a[:4321], 3.8, b[:4321], 2.5, True, True, 5.1)) and not got[4321:].any()
     h1 = rng.standard_normal((n, c)).astype(np.float16); h2 = rng.standard_normal((n, c)).astype(np.float16)
     out = torch.zeros((n, c), dtype=torch.float16, device=DEV)
     d1, d2 = to_dev(h1), to_dev(h2)
-    capi.check(L.scn_add_relu(ptr(d1), capi.DTYPE_FP16, 1.0, 0.0, ptr(d2), capi.DTYPE_FP16, 1.0, 0.0, ptr(out),
-                              capi.DTYPE_FP16, 1.0, 0, c, n, None, stream()))
+    capi.check(L.scn_add_relu(ptr(d1), capi.DTYPE_FP16, 0.0, 0.0, ptr(d2), capi.DTYPE_FP16, 0.0, 0.0, ptr(out),
+                              capi.DTYPE_FP16, 0.0, 0, c, n, None, stream()))
     torch.cuda.synchronize()
-    assert np.array_equal(out.cpu().numpy().view(np.uint16), O.add(h1, 1.0, h2, 1.0, False, False).view(np.uint16))
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), O.add(h1, 127.0, h2, 127.0, False, False).view(np.uint16))
     note("scatter dense, plain and with the fused transpose")
     dims = (2, 45, 37)
     lin = rng.choice(int(np.prod(dims)), 1500, replace=False)
@@ -331,21 +333,21 @@ def test_convert_add_and_dense():
     shape = capi.i5(1, 16, *dims)
     out = torch.full((1, 16, *dims), 3, dtype=torch.float16, device=DEV)
     d_feat, d_idx = to_dev(feat), to_dev(idx)
-    capi.check(L.scn_scatter_dense(ptr(d_feat), capi.DTYPE_FP16, 1.0, 16, 16, ptr(d_idx), 1500, None, shape, None, ptr(out), stream()))
+    capi.check(L.scn_scatter_dense(ptr(d_feat), capi.DTYPE_FP16, 0.0, 16, 16, ptr(d_idx), 1500, None, shape, None, ptr(out), stream()))
     torch.cuda.synchronize()
     assert np.array_equal(out.cpu().numpy().view(np.uint16), dense_ref.view(np.uint16))
     perm = (0, 1, 4, 2, 3)
     out = torch.full((1, 16, dims[2], dims[0], dims[1]), 3, dtype=torch.float16, device=DEV)
-    capi.check(L.scn_scatter_dense(ptr(d_feat), capi.DTYPE_FP16, 1.0, 16, 16, ptr(d_idx), 1500, None, shape,
+    capi.check(L.scn_scatter_dense(ptr(d_feat), capi.DTYPE_FP16, 0.0, 16, 16, ptr(d_idx), 1500, None, shape,
                                    capi.i5(*perm), ptr(out), stream()))
     torch.cuda.synchronize()
     assert np.array_equal(out.cpu().numpy().view(np.uint16), np.ascontiguousarray(dense_ref.transpose(perm)).view(np.uint16))
     qf = rng.integers(-127, 128, (1500, 16)).astype(np.int8)
     out = torch.zeros((1, 16, *dims), dtype=torch.float16, device=DEV)
     d_qf = to_dev(qf)
-    capi.check(L.scn_scatter_dense(ptr(d_qf), capi.DTYPE_INT8, 0.05, 16, 16, ptr(d_idx), 1500, None, shape, None, ptr(out), stream()))
+    capi.check(L.scn_scatter_dense(ptr(d_qf), capi.DTYPE_INT8, 6.35, 16, 16, ptr(d_idx), 1500, None, shape, None, ptr(out), stream()))
     torch.cuda.synchronize()
-    assert np.array_equal(out.cpu().numpy().view(np.uint16), O.scatter_dense(O.dequantize(qf, 0.05), idx, dims).view(np.uint16))
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), O.scatter_dense(O.dequantize(qf, 6.35), idx, dims).view(np.uint16))
 
 
 # ----------------------------------------------------------------------------- voxelization

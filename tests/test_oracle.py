@@ -259,47 +259,66 @@ def test_sparse_rulebook_truncation_keeps_lowest_outputs():
 
 # ----------------------------------------------------------------------------- epilogue / quantisation
 def test_requant_ties_saturation_and_two_roundings():
-    # s_out a power of two -> exact ties: rint(0.5)=0, rint(1.5)=2, rint(2.5)=2, rint(-0.5)=-0, rint(-1.5)=-2
-    acc = np.array([[1, 3, 5, -1, -3, 254, 255, 400, -400, 0]], np.int32).T.copy()  # [10,1]
-    out = O.epilogue(acc, np.array([0.25], np.float32), np.array([0.0], np.float32), False, True, 0.5)
+    # out range 254 -> r = 127/254 = 0.5 exactly: ties rint(0.5)=0, rint(1.5)=2, rint(2.5)=2, rint(-0.5)=-0, rint(-1.5)=-2
+    acc = np.array([[1, 3, 5, -1, -3, 254, 255, 400, -400, 0]], np.int32).T.copy()  # y = acc (scale 1, bias 0)
+    out = O.epilogue(acc, np.array([1.0], np.float32), np.array([0.0], np.float32), False, True, 254.0)
     assert out[:, 0].tolist() == [0, 2, 2, 0, -2, 127, 127, 127, -127, 0]
-    out = O.epilogue(acc, np.array([0.25], np.float32), np.array([0.0], np.float32), True, True, 0.5)
+    out = O.epilogue(acc, np.array([1.0], np.float32), np.array([0.0], np.float32), True, True, 254.0)
     assert out[:, 0].tolist() == [0, 2, 2, 0, 0, 127, 127, 127, 0, 0]
-    # general case against numpy fp32 arithmetic (multiply, add, divide each rounded once)
+    # general case against numpy fp32 arithmetic (multiply, add, multiply by 127/amax, each rounded once)
     rng = np.random.default_rng(7)
     acc = rng.integers(-40000, 40000, (5000, 16)).astype(np.int32)
     scale = (rng.uniform(1e-5, 1e-3, 16)).astype(np.float32)
     bias = rng.standard_normal(16).astype(np.float16).astype(np.float32)
-    s_out = np.float32(0.0371)
+    amax = np.float32(4.7117)
+    r = np.float32(127.0) / amax
     y = acc.astype(np.float32) * scale
     y = y + bias
-    q = np.clip(np.rint(np.maximum(y, 0) / s_out), -127, 127).astype(np.int8)
-    assert np.array_equal(O.epilogue(acc, scale, bias, True, True, float(s_out)), q)
+    q = np.clip(np.rint(np.maximum(y, 0) * r), -127, 127).astype(np.int8)
+    assert np.array_equal(O.epilogue(acc, scale, bias, True, True, float(amax)), q)
     assert np.array_equal(O.epilogue(acc, scale, bias, False, False).view(np.uint16), y.astype(np.float16).view(np.uint16))
     # an FMA would round differently somewhere in this sample: make sure the two-rounding rule is what runs
     y_fma = (acc.astype(np.float64) * scale.astype(np.float64) + bias.astype(np.float64)).astype(np.float32)
     assert np.any(y_fma != y)
+    # multiplying by 127/amax is not the same function as dividing by amax/127 near the rounding
+    # boundaries; the rule is the former (values built right at the boundaries tell the two apart)
+    k = np.arange(0, 127, dtype=np.float32) + np.float32(0.5)
+    yb = (k / r).astype(np.float32)
+    yb = np.concatenate([yb, np.nextafter(yb, np.float32(np.inf)), np.nextafter(yb, np.float32(-np.inf))])
+    want_mul = np.clip(np.rint(yb * r), -127, 127).astype(np.int8)
+    want_div = np.clip(np.rint(yb / (amax / np.float32(127.0))), -127, 127).astype(np.int8)
+    assert np.any(want_mul != want_div)
+    got = O.quantize_f32(yb, float(amax))
+    assert np.array_equal(got, want_mul)
 
 
 def test_quantize_dequantize_add_closed_forms():
     rng = np.random.default_rng(8)
     x = (rng.standard_normal(4000) * 3).astype(np.float16)
-    s = np.float32(0.05)
-    q = O.quantize(x, float(s))
-    assert np.array_equal(q, np.clip(np.rint(x.astype(np.float32) / s), -127, 127).astype(np.int8))
-    d = O.dequantize(q, float(s))
+    amax = np.float32(6.35)
+    r, s = np.float32(127.0) / amax, amax / np.float32(127.0)
+    q = O.quantize(x, float(amax))
+    assert np.array_equal(q, np.clip(np.rint(x.astype(np.float32) * r), -127, 127).astype(np.int8))
+    d = O.dequantize(q, float(amax))
     assert np.array_equal(d.view(np.uint16), (q.astype(np.float32) * s).astype(np.float16).view(np.uint16))
     a = rng.integers(-127, 128, 4000).astype(np.int8)
     b = rng.integers(-127, 128, 4000).astype(np.int8)
-    sa, sb, sc = np.float32(0.031), np.float32(0.027), np.float32(0.04)
-    v = np.maximum(a.astype(np.float32) * sa + b.astype(np.float32) * sb, 0)
-    assert np.array_equal(O.add(a, float(sa), b, float(sb), True, True, float(sc)),
-                          np.clip(np.rint(v / sc), -127, 127).astype(np.int8))
+    ra, rb, rc = np.float32(3.9), np.float32(3.4), np.float32(5.1)
+    v = np.maximum(a.astype(np.float32) * (ra / np.float32(127)) + b.astype(np.float32) * (rb / np.float32(127)), 0)
+    assert np.array_equal(O.add(a, float(ra), b, float(rb), True, True, float(rc)),
+                          np.clip(np.rint(v * (np.float32(127) / rc)), -127, 127).astype(np.int8))
     # relu after an int8 store == int8 store of the relu'd value (what lets Add+Relu fuse)
-    no_relu = O.add(a, float(sa), b, float(sb), False, True, float(sc))
-    assert np.array_equal(np.maximum(no_relu, 0), O.add(a, float(sa), b, float(sb), True, True, float(sc)))
-    h = O.add(x, 1.0, d, 1.0, False, False)
+    no_relu = O.add(a, float(ra), b, float(rb), False, True, float(rc))
+    assert np.array_equal(np.maximum(no_relu, 0), O.add(a, float(ra), b, float(rb), True, True, float(rc)))
+    h = O.add(x, 127.0, d, 127.0, False, False)
     assert np.array_equal(h.view(np.uint16), (x.astype(np.float32) + d.astype(np.float32)).astype(np.float16).view(np.uint16))
+    # weights: per-output-channel fake quant, multiply form
+    w = (rng.standard_normal((4, 3, 3, 3, 8)) * 0.02).astype(np.float16)
+    ranges = np.abs(w.astype(np.float32)).reshape(4, -1).max(1)
+    wq, s_w = O.quantize_weights(w, ranges)
+    ref = np.clip(np.rint(w.astype(np.float32) * (np.float32(127) / ranges)[:, None, None, None, None]), -127, 127)
+    assert np.array_equal(wq, ref.reshape(4, 27, 8).transpose(1, 0, 2).astype(np.int8)) and np.abs(wq).max() == 127
+    assert np.array_equal(s_w, ranges / np.float32(127))
 
 
 def test_scatter_dense_matches_numpy_indexing():
