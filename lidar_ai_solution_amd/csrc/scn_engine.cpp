@@ -99,7 +99,8 @@ struct CoordSet {
   uint32_t n_bound = 0;  // host-side bound of the row count for the current forward
   uint32_t cap = 0;      // allocated rows
   int grid[3] = {0, 0, 0};
-  const CoordTable* table = nullptr;  // hash of these coordinates (set once built in this forward)
+  CoordLookup lookup;                 // row look-up of these coordinates (valid once has_lookup is set in a forward)
+  bool has_lookup = false;
   CoordTable own_table;               // only for graph inputs
   int producer_rulebook = -1;         // strided rulebook that creates this set (-1: graph input)
 };
@@ -794,7 +795,7 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
       }
       c0.idx = e.in_idx;
       c0.n_bound = n;
-      c0.table = nullptr;
+      c0.has_lookup = false;
       int rc = set_count(e.in_count.as<uint32_t>(), e.dds, n, stream);
       if (rc) return rc;
       c0.n_dev = e.in_count.as<uint32_t>();
@@ -807,24 +808,28 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
       CoordSet& cs = e.coords[st.coord];
       int rc = hash_build(cs.own_table, cs.idx, cs.n_bound, cs.n_dev, cs.grid, nullptr, stream);
       if (rc) return rc;
-      cs.table = &cs.own_table;
+      cs.lookup = cs.own_table.lookup();
+      cs.has_lookup = true;
       return SCN_OK;
     }
     case StepKind::RulebookSubm: {
       RbSlot& s = *e.rulebooks[st.rulebook];
       CoordSet& cs = e.coords[s.coord_in];
-      return s.rb.build_subm(cs.idx, cs.n_bound, cs.n_dev, cs.grid, s.ks, s.dil, cs.table, stream);
+      return s.rb.build_subm(cs.idx, cs.n_bound, cs.n_dev, cs.grid, s.ks, s.dil, cs.has_lookup ? &cs.lookup : nullptr,
+                             stream);
     }
     case StepKind::RulebookSparse: {
       RbSlot& s = *e.rulebooks[st.rulebook];
       CoordSet& ci = e.coords[s.coord_in];
       CoordSet& co = e.coords[s.coord_out];
-      int rc = s.rb.build_sparse(ci.idx, ci.n_bound, ci.n_dev, ci.grid, s.ks, s.stride, s.pad, s.dil, ci.table, stream);
+      int rc = s.rb.build_sparse(ci.idx, ci.n_bound, ci.n_dev, ci.grid, s.ks, s.stride, s.pad, s.dil,
+                                 ci.has_lookup ? &ci.lookup : nullptr, stream);
       if (rc) return rc;
       co.idx = s.rb.out_indices;
       co.n_dev = s.rb.n_out_dev();
       co.n_bound = s.rb.n_bound_out;
-      co.table = &s.rb.out_table;
+      co.lookup = s.rb.out_lookup();
+      co.has_lookup = true;
       return SCN_OK;
     }
     case StepKind::Convert: {

@@ -234,12 +234,12 @@ __global__ __launch_bounds__(1024) void k_scan_blocksums(uint32_t* vals, uint32_
 }
 
 // Sparse bitmaps (fewer set bits than words): one thread per word expands its bits in rank order.
-// Optional outputs: coordinate rows, a hash table of {key -> rank}, and the per-word exclusive
-// prefix (rank of the word's first bit).  Block = 1024 threads = 1024 words.
+// Optional outputs: coordinate rows and the per-word exclusive prefix (rank of the word's first bit),
+// which together with the bitmap answers "row of this cell" (see coord_row).
+// Block = 1024 threads = 1024 words.
 __global__ __launch_bounds__(1024) void k_bitmap_expand(const uint32_t* __restrict__ bitmap,
                                                         const uint32_t* __restrict__ blockoff, Int3 grid, uint32_t cap,
-                                                        int4* coords_out, uint64_t* slots, uint32_t mask,
-                                                        uint32_t* prefix_out) {
+                                                        int4* coords_out, uint32_t* prefix_out) {
   __shared__ uint32_t scratch[17];
   const size_t t = (size_t)blockIdx.x * 1024 + threadIdx.x;
   uint32_t bits = bitmap[t];
@@ -257,7 +257,6 @@ __global__ __launch_bounds__(1024) void k_bitmap_expand(const uint32_t* __restri
       const uint32_t i0 = key / g12, rem = key - i0 * g12;
       const uint32_t i1 = rem / (uint32_t)grid.v[2], i2 = rem - i1 * (uint32_t)grid.v[2];
       coords_out[rank] = make_int4(0, (int)i0, (int)i1, (int)i2);
-      if (slots) table_insert(slots, mask, key, rank);
     }
     rank++;
   }
@@ -266,7 +265,7 @@ __global__ __launch_bounds__(1024) void k_bitmap_expand(const uint32_t* __restri
 // Dense bitmaps: one thread per cell, rank = prefix of its word + set bits below it.
 __global__ __launch_bounds__(256) void k_expand_cells(const uint32_t* __restrict__ bitmap,
                                                       const uint32_t* __restrict__ prefix, uint32_t cells, Int3 grid,
-                                                      uint32_t cap, int4* coords_out, uint64_t* slots, uint32_t mask) {
+                                                      uint32_t cap, int4* coords_out) {
   const uint32_t key = blockIdx.x * 256 + threadIdx.x;
   if (key >= cells) return;
   const uint32_t w = bitmap[key >> 5], b = key & 31;
@@ -277,7 +276,6 @@ __global__ __launch_bounds__(256) void k_expand_cells(const uint32_t* __restrict
   const uint32_t i0 = key / g12, rem = key - i0 * g12;
   const uint32_t i1 = rem / (uint32_t)grid.v[2], i2 = rem - i1 * (uint32_t)grid.v[2];
   coords_out[rank] = make_int4(0, (int)i0, (int)i1, (int)i2);
-  if (slots) table_insert(slots, mask, key, rank);
 }
 
 static size_t bitmap_words_for(const int g[3]) {
@@ -306,14 +304,33 @@ static GeomDev to_dev(const ConvGeom& g) {
   return d;
 }
 
+// Row of the voxel with linear index `key` in a tensor described by `lk`: a probe of the coordinate
+// hash (tensors in caller order), or rank = prefix[word] + popcount(bits below) in the occupancy
+// bitmap of a tensor whose rows are in canonical order (outputs of strided convolutions): two
+// independent loads, no probing loop.
+__device__ __forceinline__ int32_t coord_row(const CoordLookup& lk, uint32_t key) {
+  if (lk.bitmap) {
+    const uint32_t w = lk.bitmap[key >> 5], b = key & 31;
+    if (!((w >> b) & 1u)) return -1;
+    const uint32_t r = lk.prefix[key >> 5] + __popc(w & ((1u << b) - 1u));
+    return r < lk.rank_cap ? (int32_t)r : -1;
+  }
+  return table_lookup(lk.slots, lk.mask, key);
+}
+
 // nbr[k][o] = row of the input at  o*stride - pad + k*dilation  (or -1).  grid.y = k0; a thread
 // walks the K1*K2 offsets of its k0 plane (independent lookups, coalesced stores per offset).
 // Used for both kinds: submanifold passes stride 1 and pad = floor(K/2)*dilation.
+// Thread (0,0) also publishes the row count for the kernels that follow (n_publish, nullable).
 __global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_coords, const uint32_t* n_out_dev,
-                                                   uint32_t n_bound, GeomDev g, const uint64_t* __restrict__ slots,
-                                                   uint32_t mask, int32_t* nbr, uint32_t ld, int identity_center) {
+                                                   uint32_t n_bound, GeomDev g, CoordLookup lk, int32_t* nbr,
+                                                   uint32_t ld, int identity_center, uint32_t* n_publish) {
   const uint32_t n = eff_n(n_out_dev, n_bound);
   const uint32_t o = blockIdx.x * 256 + threadIdx.x;
+  if (n_publish && o == 0 && blockIdx.y == 0) {
+    n_publish[0] = n;
+    n_publish[1] = n;
+  }
   if (o >= n) return;
   const int k0 = blockIdx.y;
   const int4 c = out_coords[o];
@@ -323,6 +340,7 @@ __global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_
   for (int k1 = 0; k1 < g.ks[1]; ++k1) {
     const int i1 = c.z * g.st[1] - g.pd[1] + k1 * g.dl[1];
     const bool ok1 = ok0 && i1 >= 0 && i1 < g.gi[1];
+    const uint32_t line = ((uint32_t)i0 * (uint32_t)g.gi[1] + (uint32_t)i1) * (uint32_t)g.gi[2];
 #pragma unroll 3
     for (int k2 = 0; k2 < g.ks[2]; ++k2) {
       const int i2 = c.w * g.st[2] - g.pd[2] + k2 * g.dl[2];
@@ -330,8 +348,7 @@ __global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_
       if (centre0 && k1 == g.ks[1] / 2 && k2 == g.ks[2] / 2) {
         res = (int32_t)o;
       } else if (ok1 && i2 >= 0 && i2 < g.gi[2]) {
-        const uint32_t key = ((uint32_t)i0 * (uint32_t)g.gi[1] + (uint32_t)i1) * (uint32_t)g.gi[2] + (uint32_t)i2;
-        res = table_lookup(slots, mask, key);
+        res = coord_row(lk, line + (uint32_t)i2);
       }
       nbr[(size_t)((k0 * g.ks[1] + k1) * g.ks[2] + k2) * ld + o] = res;
     }
@@ -339,8 +356,9 @@ __global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_
 }
 
 // Marks every output cell reached by an input row through some kernel offset.  One thread per
-// input row; the bit is tested before the atomic so that cells reached by several inputs cost one
-// atomic, not one per input.
+// input row; per axis the (at most K) reachable output coordinates are found first, then their
+// combinations are marked.  The bit is tested before the atomic so that cells reached by several
+// inputs cost one atomic, not one per input.
 __global__ __launch_bounds__(256) void k_mark_outputs(const int4* __restrict__ in_coords, const uint32_t* n_dev,
                                                       uint32_t n_bound, GeomDev g, uint32_t* bitmap) {
   const uint32_t n = eff_n(n_dev, n_bound);
@@ -348,27 +366,30 @@ __global__ __launch_bounds__(256) void k_mark_outputs(const int4* __restrict__ i
   if (r >= n) return;
   const int4 c = in_coords[r];
   if (c.x != 0 || c.y < 0 || c.y >= g.gi[0] || c.z < 0 || c.z >= g.gi[1] || c.w < 0 || c.w >= g.gi[2]) return;
-  for (int k0 = 0; k0 < g.ks[0]; ++k0) {
-    const int t0 = c.y + g.pd[0] - k0 * g.dl[0];
-    if (t0 < 0 || t0 % g.st[0]) continue;
-    const int o0 = t0 / g.st[0];
-    if (o0 >= g.go[0]) continue;
-    for (int k1 = 0; k1 < g.ks[1]; ++k1) {
-      const int t1 = c.z + g.pd[1] - k1 * g.dl[1];
-      if (t1 < 0 || t1 % g.st[1]) continue;
-      const int o1 = t1 / g.st[1];
-      if (o1 >= g.go[1]) continue;
-      for (int k2 = 0; k2 < g.ks[2]; ++k2) {
-        const int t2 = c.w + g.pd[2] - k2 * g.dl[2];
-        if (t2 < 0 || t2 % g.st[2]) continue;
-        const int o2 = t2 / g.st[2];
-        if (o2 >= g.go[2]) continue;
-        const uint32_t key = ((uint32_t)o0 * (uint32_t)g.go[1] + (uint32_t)o1) * (uint32_t)g.go[2] + (uint32_t)o2;
+  const int cc[3] = {c.y, c.z, c.w};
+  constexpr int kMaxK = 8;  // per-axis kernel sizes above this fall back to the generic loop bound
+  int o[3][kMaxK];
+  int cnt[3] = {0, 0, 0};
+#pragma unroll
+  for (int a = 0; a < 3; ++a) {
+    const int ks = g.ks[a] < kMaxK ? g.ks[a] : kMaxK;
+    for (int k = 0; k < ks; ++k) {
+      const int t = cc[a] + g.pd[a] - k * g.dl[a];
+      if (t < 0) continue;
+      const int q = t / g.st[a];
+      if (q * g.st[a] != t || q >= g.go[a]) continue;
+      o[a][cnt[a]++] = q;
+    }
+  }
+  for (int a0 = 0; a0 < cnt[0]; ++a0)
+    for (int a1 = 0; a1 < cnt[1]; ++a1) {
+      const uint32_t line = ((uint32_t)o[0][a0] * (uint32_t)g.go[1] + (uint32_t)o[1][a1]) * (uint32_t)g.go[2];
+      for (int a2 = 0; a2 < cnt[2]; ++a2) {
+        const uint32_t key = line + (uint32_t)o[2][a2];
         const uint32_t bit = 1u << (key & 31);
         if (!(bitmap[key >> 5] & bit)) atomicOr(&bitmap[key >> 5], bit);
       }
     }
-  }
 }
 
 bool Rulebook::init(uint32_t max_in_, uint32_t max_out_, int kvol) {
@@ -385,12 +406,12 @@ bool Rulebook::init(uint32_t max_in_, uint32_t max_out_, int kvol) {
 
 static int check_geom(const int ks[3], const int st[3], const int dl[3], int kvol_cap) {
   for (int a = 0; a < 3; ++a)
-    SCN_REQUIRE(ks[a] >= 1 && st[a] >= 1 && dl[a] >= 1, SCN_ERR_INVALID, "kernel/stride/dilation must be >= 1");
+    SCN_REQUIRE(ks[a] >= 1 && ks[a] <= 8 && st[a] >= 1 && dl[a] >= 1, SCN_ERR_INVALID,
+                "kernel size must be 1..8, stride and dilation >= 1");
   SCN_REQUIRE(ks[0] * ks[1] * ks[2] <= kvol_cap, SCN_ERR_CAPACITY, "kernel volume %d exceeds the rulebook's %d",
               ks[0] * ks[1] * ks[2], kvol_cap);
   return SCN_OK;
 }
-
 
 __global__ void k_set_count(uint32_t* dst, const uint32_t* n_dev, uint32_t n_bound) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
@@ -406,18 +427,33 @@ int set_count(uint32_t* dst, const uint32_t* n_dev, uint32_t n_bound, hipStream_
   return SCN_OK;
 }
 
-static int launch_build_nbr(const Rulebook& rb, const int32_t* out_coords, uint32_t n_bound, bool identity_center,
-                            hipStream_t stream) {
-  if (n_bound == 0) return SCN_OK;
-  hipLaunchKernelGGL(k_build_nbr, dim3(ceil_div(n_bound, 256), rb.geom.ks[0]), dim3(256), 0, stream,
-                     (const int4*)out_coords, rb.n_out_dev(), n_bound, to_dev(rb.geom), rb.in_table->slots(),
-                     rb.in_table->mask, rb.nbr.as<int32_t>(), rb.ld, identity_center ? 1 : 0);
+static int launch_build_nbr(const Rulebook& rb, const int32_t* out_coords, const uint32_t* n_dev, uint32_t n_bound,
+                            bool identity_center, uint32_t* n_publish, hipStream_t stream) {
+  const uint32_t blocks = n_bound ? ceil_div(n_bound, 256) : 1;  // one block even when empty: it publishes the count
+  hipLaunchKernelGGL(k_build_nbr, dim3(blocks, rb.geom.ks[0]), dim3(256), 0, stream, (const int4*)out_coords, n_dev,
+                     n_bound, to_dev(rb.geom), rb.in_lookup, rb.nbr.as<int32_t>(), rb.ld, identity_center ? 1 : 0,
+                     n_publish);
   SCN_HIP(hipGetLastError());
   return SCN_OK;
 }
 
+CoordLookup CoordTable::lookup() const {
+  CoordLookup lk;
+  lk.slots = slots();
+  lk.mask = mask;
+  return lk;
+}
+
+CoordLookup Rulebook::out_lookup() const {
+  CoordLookup lk;
+  lk.bitmap = bitmap.as<uint32_t>();
+  lk.prefix = prefix.as<uint32_t>();
+  lk.rank_cap = n_bound_out;
+  return lk;
+}
+
 int Rulebook::build_subm(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3], const int ks[3],
-                         const int dil[3], const CoordTable* shared_in_table, hipStream_t stream) {
+                         const int dil[3], const CoordLookup* shared_lookup, hipStream_t stream) {
   const int one[3] = {1, 1, 1};
   int rc = check_geom(ks, one, dil, kvol_cap);
   if (rc) return rc;
@@ -436,19 +472,17 @@ int Rulebook::build_subm(const int32_t* idx, uint32_t n, const uint32_t* n_dev, 
   in_indices = out_indices = idx;
   n_bound_in = n_bound_out = n;
   uint32_t* cnt = counters.as<uint32_t>();
-  if (shared_in_table) {
-    in_table = shared_in_table;
-    hipLaunchKernelGGL(k_set_count, dim3(1), dim3(64), 0, stream, cnt, n_dev, n);
-    SCN_HIP(hipGetLastError());
+  if (shared_lookup) {
+    in_lookup = *shared_lookup;
   } else {
     rc = reserve_subm(true);
     if (rc) return rc;
-    rc = hash_build(own_in_table, idx, n, n_dev, grid, cnt, stream);
+    rc = hash_build(own_in_table, idx, n, n_dev, grid, nullptr, stream);
     if (rc) return rc;
-    in_table = &own_in_table;
+    in_lookup = own_in_table.lookup();
   }
   const bool odd = (ks[0] & 1) && (ks[1] & 1) && (ks[2] & 1);
-  rc = launch_build_nbr(*this, idx, n, odd, stream);
+  rc = launch_build_nbr(*this, idx, n_dev, n, odd, cnt, stream);
   if (rc) return rc;
   built = true;
   return SCN_OK;
@@ -460,14 +494,13 @@ int Rulebook::reserve_sparse(const int out_grid[3], bool need_own_in_table) {
   const size_t words = bitmap_words_for(out_grid);
   if (words > bitmap_cap_words) {
     if (!bitmap.alloc(words * 4)) return SCN_ERR_HIP;
-    if (!blocksum.alloc((words / kWordsPerBlock + 1) * 4)) return SCN_ERR_HIP;
+    if (!blocksum.alloc((words / kWordsPerBlock + 2) * 4)) return SCN_ERR_HIP;
     if (!prefix.alloc(words * 4)) return SCN_ERR_HIP;
     bitmap_cap_words = words;
   }
   bitmap_words = words;
   if (out_idx.bytes < (size_t)std::max(max_out, 1u) * 16 && !out_idx.alloc((size_t)std::max(max_out, 1u) * 16))
     return SCN_ERR_HIP;
-  if (out_table.cap < hash_capacity_for(max_out) && !out_table.alloc_for(max_out)) return SCN_ERR_HIP;
   if (need_own_in_table && own_in_table.cap < hash_capacity_for(max_in) && !own_in_table.alloc_for(max_in))
     return SCN_ERR_HIP;
   return SCN_OK;
@@ -481,7 +514,7 @@ int Rulebook::reserve_subm(bool need_own_in_table) {
 
 int Rulebook::build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3], const int ks[3],
                            const int stride[3], const int pad[3], const int dil[3],
-                           const CoordTable* shared_in_table, hipStream_t stream) {
+                           const CoordLookup* shared_lookup, hipStream_t stream) {
   int rc = check_geom(ks, stride, dil, kvol_cap);
   if (rc) return rc;
   SCN_REQUIRE(n <= max_in, SCN_ERR_CAPACITY, "sparse rulebook: %u rows exceed capacity %u", n, max_in);
@@ -508,29 +541,25 @@ int Rulebook::build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev
     uint64_t b = std::min<uint64_t>((uint64_t)n * (uint64_t)geom.kvol, vol);
     n_bound_out = (uint32_t)std::min<uint64_t>(b, max_out);
   }
-  rc = reserve_sparse(geom.grid_out, shared_in_table == nullptr);
+  rc = reserve_sparse(geom.grid_out, shared_lookup == nullptr);
   if (rc) return rc;
   const size_t words = bitmap_words;
   out_indices = out_idx.as<int32_t>();
   uint32_t* cnt = counters.as<uint32_t>();
-  // input table
-  if (shared_in_table) {
-    in_table = shared_in_table;
+  if (shared_lookup) {
+    in_lookup = *shared_lookup;
   } else {
     rc = hash_build(own_in_table, idx, n, n_dev, grid, nullptr, stream);
     if (rc) return rc;
-    in_table = &own_in_table;
+    in_lookup = own_in_table.lookup();
   }
-  // occupancy bitmap of the outputs -> ordered unique output coordinates + their hash
+  // occupancy bitmap of the outputs -> ordered unique output coordinates + per-word ranks
   rc = fill_u32(bitmap.p, 0u, words, stream);
-  if (rc) return rc;
-  out_table.mask = (uint32_t)(hash_capacity_for(n_bound_out) - 1);
-  rc = fill_u32(out_table.slots(), 0xFFFFFFFFu, ((size_t)out_table.mask + 1) * 2, stream);
   if (rc) return rc;
   const GeomDev gd = to_dev(geom);
   if (n) {
-    hipLaunchKernelGGL(k_mark_outputs, dim3(ceil_div(n, 256)), dim3(256), 0, stream, (const int4*)idx,
-                       n_dev, n, gd, bitmap.as<uint32_t>());
+    hipLaunchKernelGGL(k_mark_outputs, dim3(ceil_div(n, 256)), dim3(256), 0, stream, (const int4*)idx, n_dev, n, gd,
+                       bitmap.as<uint32_t>());
   }
   const uint32_t nblocks = (uint32_t)(words / kWordsPerBlock);
   hipLaunchKernelGGL(k_bitmap_blocksum, dim3(nblocks), dim3(256), 0, stream, bitmap.as<uint32_t>(),
@@ -540,20 +569,17 @@ int Rulebook::build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev
   const Int3 og{{geom.grid_out[0], geom.grid_out[1], geom.grid_out[2]}};
   const uint64_t cells = (uint64_t)geom.grid_out[0] * geom.grid_out[1] * geom.grid_out[2];
   if (cells <= 32ull * std::max(n_bound_out, 1u)) {
-    // dense output grid: per-word prefix, then one thread per cell
+    // dense output grid: per-word ranks, then one thread per cell
     hipLaunchKernelGGL(k_bitmap_expand, dim3(nblocks), dim3(1024), 0, stream, bitmap.as<uint32_t>(),
-                       blocksum.as<uint32_t>(), og, n_bound_out, (int4*)nullptr, (uint64_t*)nullptr, 0u,
-                       prefix.as<uint32_t>());
+                       blocksum.as<uint32_t>(), og, n_bound_out, (int4*)nullptr, prefix.as<uint32_t>());
     hipLaunchKernelGGL(k_expand_cells, dim3((unsigned)((cells + 255) / 256)), dim3(256), 0, stream,
-                       bitmap.as<uint32_t>(), prefix.as<uint32_t>(), (uint32_t)cells, og, n_bound_out, (int4*)out_idx.p,
-                       out_table.slots(), out_table.mask);
+                       bitmap.as<uint32_t>(), prefix.as<uint32_t>(), (uint32_t)cells, og, n_bound_out, (int4*)out_idx.p);
   } else {
     hipLaunchKernelGGL(k_bitmap_expand, dim3(nblocks), dim3(1024), 0, stream, bitmap.as<uint32_t>(),
-                       blocksum.as<uint32_t>(), og, n_bound_out, (int4*)out_idx.p, out_table.slots(), out_table.mask,
-                       (uint32_t*)nullptr);
+                       blocksum.as<uint32_t>(), og, n_bound_out, (int4*)out_idx.p, prefix.as<uint32_t>());
   }
   SCN_HIP(hipGetLastError());
-  rc = launch_build_nbr(*this, out_indices, n_bound_out, false, stream);
+  rc = launch_build_nbr(*this, out_indices, cnt, n_bound_out, false, nullptr, stream);
   if (rc) return rc;
   built = true;
   return SCN_OK;
@@ -1315,17 +1341,39 @@ struct DenseStrides {
   int d0, d1, d2;
 };
 
-__global__ __launch_bounds__(256) void k_scatter_dense(const void* feat, int dtype, float scale, uint32_t ld,
-                                                       const int4* __restrict__ coords, uint32_t n_bound,
+// One thread per (row, group of 8 channels): the coordinate row and 8 channels are read with one
+// vector load each; consecutive threads are consecutive rows, i.e. mostly adjacent cells of the
+// innermost dense axis, so the 8 strided stores of a wave land in 8 short contiguous runs.
+__global__ __launch_bounds__(256) void k_scatter_dense(const void* feat, int dtype, float scale, uint32_t c_total,
+                                                       uint32_t ld, const int4* __restrict__ coords, uint32_t n_bound,
                                                        const uint32_t* n_dev, DenseStrides st, _Float16* out) {
   const uint32_t n = eff_n(n_dev, n_bound);
   const uint32_t row = blockIdx.x * 256 + threadIdx.x;
   if (row >= n) return;
-  const uint32_t c = blockIdx.y;
+  const uint32_t c0 = blockIdx.y * 8;
   const int4 p = coords[row];
   if (p.x != 0 || p.y < 0 || p.y >= st.d0 || p.z < 0 || p.z >= st.d1 || p.w < 0 || p.w >= st.d2) return;
-  const float v = load_value(feat, dtype, (size_t)row * ld + c, scale, 0.f, 0.f);
-  out[c * st.sc + p.y * st.s0 + p.z * st.s1 + p.w * st.s2] = (_Float16)v;
+  _Float16* dst = out + p.y * st.s0 + p.z * st.s1 + p.w * st.s2;
+  float v[8];
+  const bool full = c0 + 8 <= c_total;
+  if (full && dtype == SCN_DTYPE_FP16 && (ld & 7) == 0) {
+    typedef _Float16 v8hh __attribute__((ext_vector_type(8)));
+    const v8hh h = *reinterpret_cast<const v8hh*>(reinterpret_cast<const _Float16*>(feat) + (size_t)row * ld + c0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (float)h[j];
+  } else if (full && dtype == SCN_DTYPE_INT8 && (ld & 7) == 0) {
+    typedef signed char v8c __attribute__((ext_vector_type(8)));
+    const v8c q = *reinterpret_cast<const v8c*>(reinterpret_cast<const signed char*>(feat) + (size_t)row * ld + c0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (float)q[j] * scale;
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      v[j] = c0 + j < c_total ? load_value(feat, dtype, (size_t)row * ld + c0 + j, scale, 0.f, 0.f) : 0.f;
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    if (c0 + j < c_total) dst[(c0 + j) * st.sc] = (_Float16)v[j];
 }
 
 int scatter_dense(const void* feat, int dtype, float range, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
@@ -1358,8 +1406,8 @@ int scatter_dense(const void* feat, int dtype, float range, uint32_t c, uint32_t
   if (n == 0) return SCN_OK;
   SCN_REQUIRE(feat && idx, SCN_ERR_INVALID, "scatter_dense: null input");
   DenseStrides st{dstride[1], dstride[2], dstride[3], dstride[4], dense_shape[2], dense_shape[3], dense_shape[4]};
-  hipLaunchKernelGGL(k_scatter_dense, dim3(ceil_div(n, 256), c), dim3(256), 0, stream, feat, dtype, scale, ld,
-                     (const int4*)idx, n, n_dev, st, (_Float16*)out);
+  hipLaunchKernelGGL(k_scatter_dense, dim3(ceil_div(n, 256), ceil_div(c, 8)), dim3(256), 0, stream, feat, dtype, scale, c,
+                     ld, (const int4*)idx, n, n_dev, st, (_Float16*)out);
   SCN_HIP(hipGetLastError());
   return SCN_OK;
 }
@@ -1609,7 +1657,7 @@ int scn_voxelizer_forward(scn_voxelizer* v, const void* points_fp16_dev, uint32_
                      (uint32_t)p.max_voxels);
   hipLaunchKernelGGL(k_bitmap_expand, dim3(nblocks), dim3(1024), 0, stream, v->bitmap.as<uint32_t>(),
                      v->blocksum.as<uint32_t>(), Int3{{g.og[0], g.og[1], g.og[2]}}, (uint32_t)p.max_voxels,
-                     (int4*)v->idx.p, (uint64_t*)nullptr, 0u, v->prefix.as<uint32_t>());
+                     (int4*)v->idx.p, v->prefix.as<uint32_t>());
   if (num_points) {
     hipLaunchKernelGGL(k_vox_assign, dim3(ceil_div(num_points, 256)), dim3(256), 0, stream, v->pkey.as<uint32_t>(),
                        num_points, v->bitmap.as<uint32_t>(), v->prefix.as<uint32_t>(), p.max_voxels,

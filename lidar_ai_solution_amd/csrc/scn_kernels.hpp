@@ -8,12 +8,23 @@ namespace scn {
 // Open-addressing coordinate hash: 64-bit slots {key (linear voxel index) << 32 | row}.
 constexpr uint64_t kEmptySlot = ~0ull;
 
+// How a kernel turns a voxel's linear index into its row: either a coordinate hash (tensors whose rows
+// are in caller order) or the occupancy bitmap + per-word ranks of a tensor in canonical order.
+struct CoordLookup {
+  const uint64_t* slots = nullptr;
+  uint32_t mask = 0;
+  const uint32_t* bitmap = nullptr;
+  const uint32_t* prefix = nullptr;
+  uint32_t rank_cap = 0;  // ranks >= rank_cap were truncated away
+};
+
 struct CoordTable {
   DevBuf buf;
   size_t cap = 0;     // allocated slots, power of two
   uint32_t mask = 0;  // slots in use - 1 (power of two <= cap), set by the last build
   bool alloc_for(uint32_t max_rows);
   uint64_t* slots() const { return buf.as<uint64_t>(); }
+  CoordLookup lookup() const;
 };
 
 size_t hash_capacity_for(uint32_t n);
@@ -34,9 +45,8 @@ struct Rulebook {
   int kvol_cap = 0;
   bool subm = false;
   ConvGeom geom{};
-  CoordTable own_in_table;    // hash of the input rows when no shared table is passed
-  CoordTable out_table;       // strided only: hash of the output rows (next stage's lookups)
-  const CoordTable* in_table = nullptr;  // the table actually used for input lookups
+  CoordTable own_in_table;    // hash of the input rows when no shared lookup is passed
+  CoordLookup in_lookup;      // what the last build used to find input rows
   DevBuf nbr;                 // int32 [kvol_cap][ld]
   uint32_t ld = 0;
   DevBuf out_idx;             // int32 [max_out][4] (strided)
@@ -53,10 +63,11 @@ struct Rulebook {
   int reserve_sparse(const int out_grid[3], bool need_own_in_table);
   int reserve_subm(bool need_own_in_table);
   int build_subm(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3], const int ks[3],
-                 const int dil[3], const CoordTable* shared_in_table, hipStream_t stream);
+                 const int dil[3], const CoordLookup* shared_lookup, hipStream_t stream);
   int build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3], const int ks[3],
-                   const int stride[3], const int pad[3], const int dil[3], const CoordTable* shared_in_table,
+                   const int stride[3], const int pad[3], const int dil[3], const CoordLookup* shared_lookup,
                    hipStream_t stream);
+  CoordLookup out_lookup() const;  // strided: rows of the output tensor from bitmap ranks
   int pairs(int32_t* pair_in, int32_t* pair_out, int64_t* offsets, uint64_t capacity, hipStream_t stream);
   const uint32_t* n_out_dev() const { return counters.as<uint32_t>(); }
 };
