@@ -907,7 +907,7 @@ constexpr int kConvMaxKvol = 27;  // largest kernel volume the workgroup kernel 
 // are in flight.  Loaded values are only touched (masked, stored) in the iteration that consumes
 // them: any earlier ALU use would make the wave wait for the load right where it was issued.
 template <int EL, int CHUNKS, int MT, int NT>
-__global__ __launch_bounds__(256) void k_conv_wg(const ConvArgs a) {
+__global__ __launch_bounds__(256, 2) void k_conv_wg(const ConvArgs a) {
   using Acc = typename Mma<EL>::Acc;
   constexpr int SPK = CHUNKS >= 4 ? CHUNKS / 4 : 1;  // K-steps per iteration
   constexpr int SLAB = SPK * MT * 64;                 // 16-byte fragments per iteration
@@ -1140,9 +1140,9 @@ static int conv_impl() {
 
 template <int EL, int CHUNKS, int MT>
 static void launch_conv_rows(const ConvArgs& a, hipStream_t stream) {
-  // Row tiles per wave.  4 for up to 64 output channels; 2 for 128: with 4 the accumulators alone take
-  // 128 registers, occupancy drops to one workgroup per CU and a 65 k-row layer becomes 257 workgroups
-  // on 256 CUs (measured 127 us against 62 us).
+  // Row tiles per wave: 4 up to 64 output channels, 2 for 128.  Measured on a 65.7 k-row 128->128
+  // layer: NT=2 58.6 us, NT=4 71.6 us (compiled for two workgroups per CU) -- with 4 the layer is only
+  // 257 workgroups, one wave per SIMD, and nothing hides the LDS and gather latency.
   constexpr int NT = MT >= 8 ? 2 : 4;
   const uint32_t rows_per_block = 4 * 16 * NT;
   constexpr int SPK = CHUNKS >= 4 ? CHUNKS / 4 : 1;

@@ -1,0 +1,158 @@
+"""The benchmark configurations at their full sizes, plus size-independent properties.  Needs a MI355X.
+
+config 2/3: CenterPoint-shaped backbone on a synthetic 250 k-point frame (fp16 tolerance / int8 bit-exact)
+config 4:   indice-generation stress, 8 frames of 50 k - 300 k points with a radial density gradient
+config 5:   BEVFusion-shaped int8 backbone end to end from 300 k points
+"""
+import numpy as np
+import pytest
+import torch
+
+from lidar_ai_solution_amd import capi, graphs, synth
+from lidar_ai_solution_amd.scn import Engine, LidarSCN, Voxelization
+from oracle import scn_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+from tests.gpu_helpers import DEV, GpuRulebook, to_dev  # noqa: E402
+from tests.test_gpu_engine import (FP16_COS, FP16_REL, GRID_XYZ, GRID_ZYX, _compare_dense, _fp16_region_override,  # noqa: E402
+                                   _oracle_calibration, _run_engine, note)
+from tests.test_gpu_stages import STAGES, _check_pairs  # noqa: E402
+
+
+def _voxelize_gpu(points, order):
+    vox = Voxelization(synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, max_points=max(300000, points.shape[0]))
+    d = to_dev(points)
+    vox.forward(d, order=order)
+    nv = vox.num_voxels()
+    from tests.gpu_helpers import copy_from_ptr
+    f = copy_from_ptr(vox.features_ptr(), (nv, 5), np.float16).cpu().numpy()
+    i = copy_from_ptr(vox.indices_ptr(), (nv, 4), np.int32).cpu().numpy()
+    vox.close()
+    return f, i
+
+
+@pytest.fixture(scope="module")
+def frame250k():
+    pts = synth.lidar_frame(seed=0, n_points=250000)
+    f, i = _voxelize_gpu(pts, "zyx")
+    rf, ri, _ = O.voxelize(pts, synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, order="zyx")
+    assert np.array_equal(i, ri) and np.array_equal(f.view(np.uint16), rf.view(np.uint16))
+    assert 114000 <= f.shape[0] <= 126000, f.shape  # "~120k non-empty voxels"
+    return f, i
+
+
+def test_config2_fp16_backbone_full_size(frame250k):
+    f, i = frame250k
+    note(f"config 2: fp16 CenterPoint-shaped backbone, {f.shape[0]} voxels")
+    g, _ = graphs.centerpoint_scn(seed=0)
+    for n in g.nodes:  # the synthetic frame grows through the strided stages: do not truncate
+        if n.op_type == "SparseConvolution":
+            n.attrs["output_bound"] = 400000
+    eng = Engine.from_graph(g, "fp16")
+    _run_engine(eng, f, i, GRID_ZYX)
+    got = eng.output(0).torch().cpu().numpy()
+    ref = O.run_graph(g, f, i, GRID_ZYX, "fp16")[g.outputs[0]]
+    maxabs, cos, refmax = _compare_dense(got, ref)
+    print(f"config 2: max-abs {maxabs:.3e} of {refmax:.3e}, cosine {cos:.6f}")
+    assert maxabs <= FP16_REL * refmax and cos >= FP16_COS
+
+
+def test_config3_int8_backbone_full_size_and_row_order_invariance(frame250k):
+    f, i = frame250k
+    note(f"config 3: int8 CenterPoint-shaped backbone, {f.shape[0]} voxels, default output_bound (stage 1 truncates)")
+    g16, tags = graphs.centerpoint_scn(seed=0)
+    amax = _oracle_calibration(g16, f, i, GRID_ZYX)
+    g8, tags8 = graphs.centerpoint_scn(seed=0)
+    graphs.apply_int8_plan(g8, tags8, amax, "centerpoint")
+    keep = Engine.from_graph(g8, "int8", keep_all=True)
+    _run_engine(keep, f, i, GRID_ZYX)
+    rec = {}
+    O.run_graph(g8, f, i, GRID_ZYX, "int8", rec, override=_fp16_region_override(g8, keep))
+    want = rec[g8.nodes[-1].name]["out"]
+    # every int8 conv's accumulators at full size
+    import ctypes as C
+    hip = capi.hip_runtime()
+    hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+    prec = O.node_precisions(g8, "int8")
+    nconv = 0
+    for n in g8.nodes:
+        if n.op_type == "SparseConvolution" and prec[n.name][0] == "int8":
+            view, acc_ptr = keep.tensor(n.outputs[0])
+            a = rec[n.name]["acc"]
+            acc = torch.empty(a.shape, dtype=torch.int32, device=DEV)
+            torch.cuda.synchronize()
+            assert hip.hipMemcpy(C.c_void_p(acc.data_ptr()), C.c_void_p(acc_ptr), acc.numel() * 4, 3) == 0
+            assert np.array_equal(acc.cpu().numpy(), a), n.name
+            feats, _ = view.torch()
+            assert np.array_equal(feats.cpu().numpy()[:, :a.shape[1]], rec[n.name]["out"]), n.name
+            nconv += 1
+    assert nconv == 18
+    eng = Engine.from_graph(g8, "int8")
+    _run_engine(eng, f, i, GRID_ZYX)
+    got = eng.output(0).torch().cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    note("property: the dense output does not depend on the order of the input rows (int8 path, bit for bit)")
+    perm = np.random.default_rng(1).permutation(f.shape[0])
+    _run_engine(eng, f[perm], i[perm], GRID_ZYX)
+    got2 = eng.output(0).torch().cpu().numpy()
+    assert np.array_equal(got2.view(np.uint16), got.view(np.uint16))
+    note("property: replaying the same frame gives the same bits (no state leaks between forwards)")
+    _run_engine(eng, f, i, GRID_ZYX)
+    assert np.array_equal(eng.output(0).torch().cpu().numpy().view(np.uint16), got.view(np.uint16))
+
+
+def test_config4_indice_generation_stress():
+    """8 seeded frames, 50 k - 300 k points, near range 10x denser than far range: voxel coordinates,
+    output coordinates and rulebook pairs of every stage are bit-exact; hash / offset statistics reported."""
+    sizes = [50000, 85000, 120000, 160000, 200000, 240000, 270000, 300000]
+    for s, npts in enumerate(sizes):
+        pts = synth.gradient_frame(seed=40 + s, n_points=npts)
+        f, idx = _voxelize_gpu(pts, "zyx")
+        rf, ri, _ = O.voxelize(pts, synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, order="zyx")
+        assert np.array_equal(idx, ri) and np.array_equal(f.view(np.uint16), rf.view(np.uint16))
+        grid = list(GRID_ZYX)
+        empties = []
+        for st in range(4):
+            n = idx.shape[0]
+            note(f"config 4 frame {s} ({npts} points) stage {st}: {n} rows")
+            d_idx = to_dev(idx)
+            sub = GpuRulebook(n, n, 27)
+            sub.build_subm(d_idx, n, grid, (3, 3, 3))
+            ref = O.rulebook_subm(idx, grid, (3, 3, 3))
+            _check_pairs(sub, ref)
+            empties.append(int((np.diff(ref.offsets) == 0).sum()))
+            k, sd, p = STAGES[st]
+            sp = GpuRulebook(n, 400000, int(np.prod(k)))
+            sp.build_sparse(d_idx, n, grid, k, sd, p)
+            ref2 = O.rulebook_sparse(idx, grid, k, sd, p, max_out=400000)
+            assert sp.n_out() == ref2.n_out and np.array_equal(sp.out_indices(), ref2.out_indices)
+            _check_pairs(sp, ref2)
+            idx, grid = ref2.out_indices, ref2.out_grid
+        cap = capi.lib().scn_hash_capacity_for(f.shape[0])
+        print(f"frame {s}: {npts} points -> {f.shape[0]} voxels, input hash load factor {f.shape[0] / cap:.2f}, "
+              f"empty SubM offsets per stage {empties}")
+
+
+def test_config5_bevfusion_int8_end_to_end():
+    note("config 5: 300 k points, dt in U[0,0.5] -> voxelize (xyz) -> BEVFusion-shaped int8 backbone -> BEV")
+    pts = synth.lidar_frame(seed=5, n_points=300000, dt_max=0.5)
+    rf, ri, _ = O.voxelize(pts, synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, order="xyz")
+    g16, tags = graphs.bevfusion_scn(seed=2)
+    amax = _oracle_calibration(g16, rf, ri, GRID_XYZ)
+    g8, tags8 = graphs.bevfusion_scn(seed=2)
+    graphs.apply_int8_plan(g8, tags8, amax, "bevfusion")
+    keep = Engine.from_graph(g8, "int8", keep_all=True)
+    _run_engine(keep, rf, ri, GRID_XYZ)
+    rec = {}
+    O.run_graph(g8, rf, ri, GRID_XYZ, "int8", rec, override=_fp16_region_override(g8, keep))
+    want = rec[g8.nodes[-1].name]["out"]
+    vox = Voxelization(synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, max_voxels=160000, max_points=300000)
+    scn = LidarSCN(g8, vox, order="xyz", precision="int8")
+    out = scn.forward(to_dev(pts))
+    torch.cuda.synchronize()
+    assert vox.num_voxels() == rf.shape[0]
+    got = out.torch().cpu().numpy()
+    assert got.shape == (1, 256, 180, 180) and got.dtype == np.float16
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    assert np.count_nonzero(got) > 1000000
