@@ -1240,8 +1240,8 @@ int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, cons
   if (w.precision == SCN_PRECISION_INT8)
     SCN_REQUIRE(io.x_dynamic_range > 0.f, SCN_ERR_INVALID, "conv: int8 input needs x_dynamic_range > 0");
   {
-    static const int dbg = getenv("SCN_CONV_DEBUG") ? atoi(getenv("SCN_CONV_DEBUG")) : 0;
-    a.debug = dbg;
+    const char* dbg = getenv("SCN_CONV_DEBUG");
+    a.debug = dbg ? atoi(dbg) : 0;
   }
   bool ok = w.precision == SCN_PRECISION_INT8 ? dispatch_chunks<0>(w.chunks, w.mtiles, a, stream)
                                                : dispatch_chunks<1>(w.chunks, w.mtiles, a, stream);
