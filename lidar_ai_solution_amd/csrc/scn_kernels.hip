@@ -22,6 +22,8 @@ namespace scn {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 // --------------------------------------------------------------------------------------------
@@ -689,6 +691,7 @@ struct ConvArgs {
   float a_rq_s, a_rq_r;     // re-quantisation of an fp16 operand by an int8 Add (0 = none)
   float b_rq_s, b_rq_r;
   int relu2;
+  const char* zrow;  // >= 256 bytes of zeros (gather source of lanes without a neighbour)
   int debug;  // measurement knob: 1 = no gathers, 2 = no weight slab loads, 8 = no epilogue, 16 = no main loop
 };
 
@@ -1032,14 +1035,15 @@ __global__ __launch_bounds__(256, 2) void k_conv_wg(const ConvArgs a) {
         for (int u = 0; u < NT; ++u) bm[u] = (sv && rvalid[u] && idx0[u] >= 0) ? bcur[ss][u] : vzero;
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
-          const v4i av = la[(ss * MT + t) * 64];
+          v4i av = vzero;
+          if (!(a.debug & 32)) av = la[(ss * MT + t) * 64];
 #pragma unroll
           for (int u = 0; u < NT; ++u) acc[t][u] = Mma<EL>::run(av, bm[u], acc[t][u]);
         }
       }
     }
     if (more) SCN_STORE_SLAB((it + 1) & 1);
-    __syncthreads();
+    if (!(a.debug & 64)) __syncthreads();
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
       idx0[u] = idx1[u];
@@ -1061,6 +1065,440 @@ __global__ __launch_bounds__(256, 2) void k_conv_wg(const ConvArgs a) {
 #pragma unroll
     for (int t = 0; t < MT; ++t) epilogue_store<EL>(a, rows[u], t * 16 + lg * 4, acc[t][u]);
   }
+}
+
+// --------------------------------------------------------------------------------------------
+// 32x32 MFMA variant (output channels >= 32).
+// Measured issue rates on MI355X (independent accumulators, 4 waves per SIMD): v_mfma_i32_32x32x32_i8
+// 4.77 POP/s and v_mfma_f32_32x32x16_f16 2.39 PFLOP/s, against 2.7 POP/s / 1.35 PFLOP/s for the
+// 16x16x64 / 16x16x32 forms: only the 32x32 forms reach the matrix peak, so wide layers use them.
+// Operand mapping (wave64):  A (32 x K): lane l supplies row m = l % 32, the 16 bytes of K-half l / 32
+//                            B (K x 32): lane l supplies col n = l % 32, the 16 bytes of K-half l / 32
+//                            D (32 x 32): lane l holds col n = l % 32, rows 8 * (j / 4) + 4 * (l / 32) + j % 4
+// Rows of A are output channels, columns of B voxels; K-step s consumes chunks 2s and 2s+1 of the
+// (offset, chunk) sequence.  Otherwise the pipeline is that of k_conv_wg.
+template <int EL>
+struct Mma32;
+template <>
+struct Mma32<0> {
+  using Acc = v16i;
+  using Acc4 = v4i;
+  static __device__ __forceinline__ Acc run(const v4i a, const v4i b, Acc c) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma32<1> {
+  using Acc = v16f;
+  using Acc4 = v4f;
+  static __device__ __forceinline__ Acc run(const v4i a, const v4i b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+};
+
+template <int EL, int CHUNKS, int MT, int NT>
+__global__ __launch_bounds__(256, 2) void k_conv32(const ConvArgs a) {
+  using Acc = typename Mma32<EL>::Acc;
+  using Acc4 = typename Mma32<EL>::Acc4;
+  constexpr int IPO = CHUNKS > 8 ? CHUNKS / 8 : 1;            // iterations per kernel offset
+  constexpr int SPK = CHUNKS >= 2 ? (CHUNKS / 2) / IPO : 1;   // K-steps per iteration
+  constexpr int SLAB = SPK * MT * 64;                         // 16-byte fragments per iteration
+  constexpr int WPT = (SLAB + 255) / 256;
+  constexpr int R = 128 * NT;                                 // output rows per workgroup
+  __shared__ v4i lds[3][SLAB];
+  __shared__ int32_t lidx[kConvMaxKvol * R];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int ln = lane & 31, lh = lane >> 5;
+  const uint32_t n = eff_n(a.n_out_dev, a.n_bound);
+  uint32_t tile;
+  if (!xcd_tile(n, R, &tile)) return;
+  const uint32_t row0 = (tile * 4 + wave) * (32 * NT);
+  {
+    const uint32_t tile_row0 = tile * R;
+    const int total = a.kvol * R;
+    for (int base = 0; base < total; base += 256 * 8) {
+      int32_t tmp[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int f = base + j * 256 + tid;
+        const int k = f / R, r = f - k * R;
+        const bool v = f < total && tile_row0 + r < n;
+        tmp[j] = v ? a.nbr[(size_t)k * a.nbr_ld + tile_row0 + r] : -1;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int f = base + j * 256 + tid;
+        if (f < total) lidx[f] = tmp[j];
+      }
+    }
+  }
+  __syncthreads();
+  const int32_t* __restrict__ my_idx = lidx + wave * (32 * NT) + ln;
+  const int iters = CHUNKS >= 2 ? a.kvol * IPO : (a.kvol + 1) / 2;
+  const char* __restrict__ xb = a.x;
+  const v4i* __restrict__ wsrc = reinterpret_cast<const v4i*>(a.wfrag);
+  const uint32_t ldb = a.x_ld_bytes;
+  uint32_t rows[NT];
+#pragma unroll
+  for (int u = 0; u < NT; ++u) rows[u] = row0 + u * 32 + ln;
+
+  Acc acc[MT][NT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int u = 0; u < NT; ++u)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[t][u][j] = 0;
+
+  // Software pipeline, steady state of iteration i:
+  //   issue   weight slab i+2 -> registers, gathers of i+1 -> registers, neighbour rows of i+2 <- LDS
+  //   compute MFMAs of i on the gathers issued during i-1 and the slab in LDS buffer i % 2
+  //   store   weight slab i+1 (loaded during i-1) -> LDS buffer (i+1) % 2, barrier
+  // Nothing in the loop is conditional and no loaded register is copied: the wave's memory counter
+  // retires loads in order, so a branch around a load (or a register move of a load's result)
+  // makes the compiler wait for *all* outstanding loads where the result is first touched, and the
+  // prefetch distance collapses to zero.  Hence the loop is unrolled by two with ping-pong register
+  // sets, and iterations past the end re-load the last slab / row 0 instead of skipping the loads.
+  int32_t idx0[NT], idx1[NT], idx2[NT];
+  v4i bA[SPK][NT], bB[SPK][NT];
+  v4i wA[WPT], wB[WPT];
+  const v4i vzero = {0, 0, 0, 0};
+  const int last = iters - 1;
+
+// does this lane's slot of iteration IT exist (known without any load), and its kernel offset
+#define SCN_SLOT_VALID(IT) ((IT) < iters && (CHUNKS >= 2 || 2 * (IT) + lh < a.kvol))
+#define SCN_SLOT_K(IT) (CHUNKS >= 2 ? (IT) / IPO : 2 * (IT) + lh)
+// neighbour rows of iteration IT from the LDS copy (rows beyond n hold -1 there)
+#define SCN_LOAD_IDX(IT, DST)                                                              \
+  {                                                                                        \
+    const int k_ = SCN_SLOT_VALID(IT) ? SCN_SLOT_K(IT) : 0;                                \
+    _Pragma("unroll") for (int u = 0; u < NT; ++u) DST[u] = my_idx[k_ * R + u * 32];       \
+  }
+// unconditional gathers (row 0 for lanes without a neighbour); masked to zero when consumed
+#define SCN_GATHER(IT, IDX, DST)                                                           \
+  {                                                                                        \
+    const bool sv_ = SCN_SLOT_VALID(IT);                                                   \
+    const int sub_ = CHUNKS >= 2 ? ((IT) % IPO) * (2 * SPK) : 0;                           \
+    _Pragma("unroll") for (int u = 0; u < NT; ++u) {                                       \
+      const bool ok_ = sv_ && IDX[u] >= 0;                                                 \
+      const char* p_ = xb + (size_t)(ok_ ? (uint32_t)IDX[u] : 0u) * ldb;                   \
+      _Pragma("unroll") for (int ss = 0; ss < SPK; ++ss) {                                 \
+        const int c_ = CHUNKS >= 2 ? sub_ + 2 * ss + lh : 0;                               \
+        DST[ss][u] = *reinterpret_cast<const v4i*>(p_ + c_ * 16);                          \
+      }                                                                                    \
+    }                                                                                      \
+  }
+#define SCN_LOAD_SLAB(IT, W)                                                               \
+  {                                                                                        \
+    const int it_ = (IT) < last ? (IT) : last;                                             \
+    _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                                      \
+      const int f_ = tid + j * 256;                                                        \
+      W[j] = wsrc[(size_t)it_ * SLAB + ((SLAB % 256 == 0 || f_ < SLAB) ? f_ : 0)];         \
+    }                                                                                      \
+  }
+#define SCN_STORE_SLAB(BUF, W)                                                             \
+  {                                                                                        \
+    _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                                      \
+      const int f_ = tid + j * 256;                                                        \
+      if (SLAB % 256 == 0 || f_ < SLAB) lds[BUF][f_] = W[j];                               \
+    }                                                                                      \
+  }
+// one iteration: CUR / NXT / NN = LDS buffers of slabs IT, IT+1, IT+2 (indices mod 3)
+#define SCN_ITER(IT, BC, BN, WC, WN)                                                       \
+  {                                                                                        \
+    SCN_LOAD_IDX((IT) + 2, idx2);                                                          \
+    SCN_LOAD_SLAB((IT) + 3, WN);                                                           \
+    SCN_GATHER((IT) + 1, idx1, BN);                                                        \
+    __builtin_amdgcn_sched_barrier(0);                                                     \
+    const bool sv = SCN_SLOT_VALID(IT);                                                    \
+    const int nxt_ = cur == 2 ? 0 : cur + 1;                                               \
+    const int nn_ = nxt_ == 2 ? 0 : nxt_ + 1;                                              \
+    const v4i* la = &lds[nxt_][0] + lane;                                                  \
+    _Pragma("unroll") for (int ss = 0; ss < SPK; ++ss) {                                   \
+      v4i bm[NT];                                                                          \
+      _Pragma("unroll") for (int u = 0; u < NT; ++u)                                       \
+        bm[u] = (sv && idx0[u] >= 0) ? BC[ss][u] : vzero;                                  \
+      _Pragma("unroll") for (int t = 0; t < MT; ++t)                                       \
+        _Pragma("unroll") for (int u = 0; u < NT; ++u)                                     \
+          acc[t][u] = Mma32<EL>::run(af[ss][t], bm[u], acc[t][u]);                         \
+      /* the same K-step of the next iteration, from the slab stored one iteration ago */  \
+      _Pragma("unroll") for (int t = 0; t < MT; ++t) af[ss][t] = la[(ss * MT + t) * 64];   \
+      __builtin_amdgcn_sched_barrier(0); /* keep the refill here: the scheduler sinks it to its use */ \
+    }                                                                                      \
+    SCN_STORE_SLAB(nn_, WC);                                                               \
+    __syncthreads();                                                                       \
+    cur = nxt_;                                                                            \
+    _Pragma("unroll") for (int u = 0; u < NT; ++u) {                                       \
+      idx0[u] = idx1[u];                                                                   \
+      idx1[u] = idx2[u];                                                                   \
+    }                                                                                      \
+  }
+
+  v4i af[SPK][MT];  // A fragments of the current iteration, refilled one iteration ahead
+  int cur = 0;
+  SCN_LOAD_IDX(0, idx0);
+  SCN_LOAD_IDX(1, idx1);
+  SCN_LOAD_SLAB(0, wA);
+  SCN_LOAD_SLAB(1, wB);
+  SCN_GATHER(0, idx0, bA);
+  SCN_STORE_SLAB(0, wA);
+  SCN_STORE_SLAB(1, wB);
+  SCN_LOAD_SLAB(2, wB);
+  __syncthreads();
+#pragma unroll
+  for (int ss = 0; ss < SPK; ++ss)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) af[ss][t] = lds[0][(ss * MT + t) * 64 + lane];
+  int it = 0;
+  for (; it + 1 < iters; it += 2) {
+    SCN_ITER(it, bA, bB, wB, wA);
+    SCN_ITER(it + 1, bB, bA, wA, wB);
+  }
+  if (it < iters) SCN_ITER(it, bA, bB, wB, wA);
+#undef SCN_SLOT_VALID
+#undef SCN_SLOT_K
+#undef SCN_LOAD_IDX
+#undef SCN_GATHER
+#undef SCN_LOAD_SLAB
+#undef SCN_STORE_SLAB
+#undef SCN_ITER
+  if (a.debug & 8) return;
+  const int cout_pad = (a.cout + 15) & ~15;
+#pragma unroll
+  for (int u = 0; u < NT; ++u) {
+    if (rows[u] >= n) continue;
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int co = t * 32 + g * 8 + lh * 4;
+        if (co >= cout_pad) continue;
+        const Acc4 piece = {acc[t][u][4 * g], acc[t][u][4 * g + 1], acc[t][u][4 * g + 2], acc[t][u][4 * g + 3]};
+        epilogue_store<EL>(a, rows[u], co, piece);
+      }
+  }
+}
+
+// --------------------------------------------------------------------------------------------
+// LDS-staged gather kernel (32x32 MFMA, output channels >= 32).
+// What bounds the register-gather kernels above is the vector-memory path, not the matrix cores: a
+// gather in MFMA operand order (32 rows x 2 lanes x 16 B) costs ~97 cycles of a CU's texture pipe per
+// instruction, one whose 8 adjacent lanes read one row's 128 contiguous bytes ~35 (both measured,
+// L2-resident table).  So rows are gathered in the memory-friendly order, straight into LDS
+// (global_load_lds_dwordx4: no registers, no masking -- lanes without a neighbour read a row of zeros),
+// two iterations ahead, and the MFMA B operand is read back from LDS.  Hardware places lane l's 16 bytes
+// at base + 16 l, so the bank-conflict-free read order is obtained by permuting which chunk of its row
+// a lane fetches: position p of a row holds chunk p ^ swz(row).
+//   iteration     = 4 K-steps = 4 KB of gathered rows per wave (32 rows x 8 chunks, or G = 8 / SEG
+//                   kernel offsets of SEG-chunk rows) and a weight slab of 4 * MT fragments
+//   weight slabs  = global -> registers -> LDS (triple buffered), A fragments of iteration i+1 are read
+//                   from LDS during iteration i
+//   per iteration = one barrier; each wave consumes only rows it gathered itself, so gathers need a
+//                   wait on the wave's own memory counter, not a barrier
+template <int EL, int CHUNKS, int MT, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void k_conv_lds(const ConvArgs a) {
+  using Acc = typename Mma32<EL>::Acc;
+  using Acc4 = typename Mma32<EL>::Acc4;
+  constexpr int THREADS = 64 * WAVES;
+  constexpr int SEG = CHUNKS < 8 ? CHUNKS : 8;   // chunks gathered per row and iteration
+  constexpr int IPO = CHUNKS / SEG;              // iterations per kernel offset (rows wider than 128 B)
+  constexpr int G = 8 / SEG;                     // kernel offsets per iteration
+  constexpr int RP = 8 / SEG;                    // rows per 128 bytes of a gathered stage
+  constexpr int SLAB = 4 * MT * 64;              // 16-byte weight fragments per iteration
+  constexpr int WPT = (SLAB + THREADS - 1) / THREADS;
+  constexpr int R = 32 * WAVES;                  // output rows per workgroup
+  __shared__ v4i lds[3][SLAB];
+  __shared__ v4i ring[2][WAVES][256];            // gathered rows: two stages of 4 KB per wave
+  __shared__ int32_t lidx[kConvMaxKvol * R];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int ln = lane & 31, lh = lane >> 5;
+  const uint32_t n = eff_n(a.n_out_dev, a.n_bound);
+  uint32_t tile;
+  if (!xcd_tile(n, R, &tile)) return;
+  const uint32_t row0 = (tile * WAVES + wave) * 32;
+  {
+    const uint32_t tile_row0 = tile * R;
+    const int total = a.kvol * R;
+    for (int base = 0; base < total; base += THREADS * 8) {
+      int32_t tmp[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int f = base + j * THREADS + tid;
+        const int k = f / R, r = f - k * R;
+        const bool v = f < total && tile_row0 + r < n;
+        tmp[j] = v ? a.nbr[(size_t)k * a.nbr_ld + tile_row0 + r] : -1;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int f = base + j * THREADS + tid;
+        if (f < total) lidx[f] = tmp[j];
+      }
+    }
+  }
+  __syncthreads();
+  const int iters = IPO > 1 ? a.kvol * IPO : (a.kvol + G - 1) / G;
+  const int last = iters - 1;
+  const char* __restrict__ xb = a.x;
+  const char* __restrict__ zrow = a.zrow;
+  const v4i* __restrict__ wsrc = reinterpret_cast<const v4i*>(a.wfrag);
+  const uint32_t ldb = a.x_ld_bytes;
+
+  // this lane's four gather slots: element e = 64 q + lane of the stage's [G][32 rows][SEG] array
+  int g_row[4], g_off[4], g_chunk[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int e = q * 64 + lane;
+    const int row = (e / SEG) % 32, c = e % SEG;
+    g_off[q] = e / (32 * SEG);
+    g_row[q] = row;
+    g_chunk[q] = c ^ ((row / RP) % SEG);
+  }
+  // this lane's B-operand read positions (16-byte units inside a stage) for the 4 K-steps
+  int b_pos[4];
+#pragma unroll
+  for (int ss = 0; ss < 4; ++ss) {
+    if (SEG >= 2) {
+      constexpr int SPO = SEG >= 2 ? SEG / 2 : 1;
+      const int g = ss / SPO, cl = 2 * (ss % SPO) + lh;
+      b_pos[ss] = (g * 32 + ln) * SEG + (cl ^ ((ln / RP) % SEG));
+    } else {
+      b_pos[ss] = (2 * ss + lh) * 32 + ln;
+    }
+  }
+  const int32_t* __restrict__ my_idx = lidx + wave * 32;
+
+  Acc acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[t][j] = 0;
+
+// neighbour rows of this lane's four gather slots of iteration IT (-1: none)
+#define SCN_GATHER_IDX(IT, GI)                                                                  \
+  {                                                                                             \
+    _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                             \
+      const int k_ = IPO > 1 ? (IT) / IPO : (IT) * G + g_off[q];                                \
+      const bool kv_ = (IT) < iters && k_ < a.kvol;                                             \
+      GI[q] = my_idx[(kv_ ? k_ : 0) * R + g_row[q]];                                            \
+    }                                                                                           \
+  }
+// gathers of iteration IT into ring stage STG: lanes whose slot has no neighbour (or lies beyond the
+// kernel volume / the iteration count) read the row of zeros
+#define SCN_GATHER(IT, STG, GI)                                                                 \
+  {                                                                                             \
+    _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                             \
+      const int k_ = IPO > 1 ? (IT) / IPO : (IT) * G + g_off[q];                                \
+      const bool kv_ = (IT) < iters && k_ < a.kvol;                                             \
+      const int cg_ = (IPO > 1 ? ((IT) % IPO) * 8 : 0) + g_chunk[q];                            \
+      const char* p_ = (kv_ && GI[q] >= 0) ? xb + (size_t)(uint32_t)GI[q] * ldb + cg_ * 16 : zrow + cg_ * 16; \
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)p_,       \
+                                       (__attribute__((address_space(3))) void*)&ring[STG][wave][q * 64], 16, 0, 0); \
+    }                                                                                           \
+  }
+#define SCN_LOAD_SLAB(IT, W)                                                                    \
+  {                                                                                             \
+    const int it_ = (IT) < last ? (IT) : last;                                                  \
+    _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                                           \
+      const int f_ = tid + j * THREADS;                                                         \
+      W[j] = wsrc[(size_t)it_ * SLAB + ((SLAB % THREADS == 0 || f_ < SLAB) ? f_ : 0)];          \
+    }                                                                                           \
+  }
+#define SCN_STORE_SLAB(BUF, W)                                                                  \
+  {                                                                                             \
+    _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                                           \
+      const int f_ = tid + j * THREADS;                                                         \
+      if (SLAB % THREADS == 0 || f_ < SLAB) lds[BUF][f_] = W[j];                                \
+    }                                                                                           \
+  }
+// Waits are explicit in the loop: the wave's memory counter retires loads in order, so "at most N
+// outstanding" identifies exactly which older load has landed.  Issue order per iteration IT:
+//   slab load S(IT) (WPT loads, top)  ->  gathers G(IT+2) (4 loads, after K-step 0)
+#define SCN_WAIT_VM(N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory")
+// Barrier that waits for the wave's LDS traffic except the KEEP newest operations (LDS completes in
+// order).  __syncthreads() would also drain the memory counter, i.e. every gather in flight.
+#define SCN_LDS_BARRIER(KEEP) asm volatile("s_waitcnt lgkmcnt(%0)\n\ts_barrier" ::"n"(KEEP) : "memory")
+// one iteration; STG = ring stage of its gathered rows (IT % 2), already read into BC
+#define SCN_ITER(IT, STG, BC, BN, WC, WN)                                                       \
+  {                                                                                             \
+    SCN_LOAD_SLAB((IT) + 3, WN);                                                                \
+    int32_t gi[4];                                                                              \
+    SCN_GATHER_IDX((IT) + 2, gi);                                                               \
+    const int nxt_ = cur == 2 ? 0 : cur + 1;                                                    \
+    const int nn_ = nxt_ == 2 ? 0 : nxt_ + 1;                                                   \
+    SCN_WAIT_VM(WPT + 4); /* S(IT-1) landed; younger: G(IT+1), S(IT) */                         \
+    SCN_STORE_SLAB(nn_, WC);                                                                    \
+    __builtin_amdgcn_sched_barrier(0);                                                          \
+    const v4i* la = &lds[nxt_][0] + lane;                                                       \
+    _Pragma("unroll") for (int ss = 0; ss < 4; ++ss) {                                          \
+      _Pragma("unroll") for (int t = 0; t < MT; ++t)                                            \
+        acc[t] = Mma32<EL>::run(af[ss][t], BC[ss], acc[t]);                                     \
+      _Pragma("unroll") for (int t = 0; t < MT; ++t) af[ss][t] = la[(ss * MT + t) * 64];        \
+      /* stage STG was read into BC during the previous iteration: free for the gathers of IT+2 */ \
+      if (ss == 0) SCN_GATHER((IT) + 2, STG, gi);                                               \
+      if (ss == 1) {                                                                            \
+        SCN_WAIT_VM(WPT + 4); /* G(IT+1) landed; younger: S(IT), G(IT+2) */                     \
+        _Pragma("unroll") for (int s2 = 0; s2 < 4; ++s2) BN[s2] = ring[(STG) ^ 1][wave][b_pos[s2]]; \
+      }                                                                                         \
+      __builtin_amdgcn_sched_barrier(0);                                                        \
+    }                                                                                           \
+    SCN_LDS_BARRIER(MT); /* all but the last MT fragment refills */                             \
+    cur = nxt_;                                                                                 \
+  }
+
+  v4i wA[WPT], wB[WPT];
+  v4i af[4][MT];
+  v4i bfA[4], bfB[4];
+  int cur = 0;
+  {
+    int32_t g0[4], g1[4];
+    SCN_GATHER_IDX(0, g0);
+    SCN_GATHER_IDX(1, g1);
+    SCN_LOAD_SLAB(0, wA);
+    SCN_LOAD_SLAB(1, wB);
+    SCN_GATHER(0, 0, g0);
+    SCN_WAIT_VM(4);
+    SCN_STORE_SLAB(0, wA);
+    SCN_STORE_SLAB(1, wB);
+    __builtin_amdgcn_sched_barrier(0);
+    SCN_LOAD_SLAB(2, wB);
+    SCN_GATHER(1, 1, g1);
+  }
+  SCN_LDS_BARRIER(0);
+#pragma unroll
+  for (int ss = 0; ss < 4; ++ss)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) af[ss][t] = lds[0][(ss * MT + t) * 64 + lane];
+  SCN_WAIT_VM(WPT + 4);  // G(0) landed; younger: S(2), G(1)
+#pragma unroll
+  for (int ss = 0; ss < 4; ++ss) bfA[ss] = ring[0][wave][b_pos[ss]];
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  int it = 0;
+  for (; it + 1 < iters; it += 2) {
+    SCN_ITER(it, 0, bfA, bfB, wB, wA);
+    SCN_ITER(it + 1, 1, bfB, bfA, wA, wB);
+  }
+  if (it < iters) SCN_ITER(it, 0, bfA, bfB, wB, wA);
+#undef SCN_WAIT_VM
+#undef SCN_GATHER_IDX
+#undef SCN_LDS_BARRIER
+#undef SCN_GATHER
+#undef SCN_LOAD_SLAB
+#undef SCN_STORE_SLAB
+#undef SCN_ITER
+  const uint32_t row = row0 + ln;
+  if (row >= n) return;
+  const int cout_pad = (a.cout + 15) & ~15;
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int co = t * 32 + g * 8 + lh * 4;
+      if (co >= cout_pad) continue;
+      const Acc4 piece = {acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
+      epilogue_store<EL>(a, row, co, piece);
+    }
 }
 
 bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* ranges, const uint16_t* bias_fp16,
@@ -1118,6 +1556,42 @@ bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* 
           }
         }
       }
+  // 32x32 MFMA order for layers with more than 16 output channels: [step][mtile32][lane] x 16 bytes,
+  // lane l = channel 32 t + l % 32, K-half l / 32; K-step s holds chunks 2s, 2s+1 of the sequence
+  if (mtiles >= 2) {
+    mtiles32 = (cout + 31) / 32;
+    if (mtiles32 == 3) mtiles32 = 4;  // kernels exist for 1, 2 and 4 tiles; the fourth is zero weights
+    steps32 = 4 * ((kvol * chunks + 7) / 8);  // whole iterations of 4 K-steps, zero weights beyond the volume
+    std::vector<uint8_t> f32((size_t)steps32 * mtiles32 * 64 * 16, 0);
+    for (int s = 0; s < steps32; ++s)
+      for (int t = 0; t < mtiles32; ++t)
+        for (int l = 0; l < 64; ++l) {
+          const int g = 2 * s + l / 32;
+          if (g >= kvol * chunks) continue;
+          const int k = g / chunks, c = g % chunks;
+          const int co = 32 * t + l % 32;
+          if (co >= cout) continue;
+          uint8_t* dst = &f32[((size_t)(s * mtiles32 + t) * 64 + l) * 16];
+          for (int e = 0; e < epc; ++e) {
+            const int ci = c * epc + e;
+            if (ci >= cin) break;
+            const uint16_t hb = w_fp16[((size_t)co * kvol + k) * cin + ci];
+            if (prec == SCN_PRECISION_INT8) {
+              float q = rintf(half_bits_to_float(hb) * (127.f / ranges[co]));
+              if (!(q >= -127.f)) q = -127.f;
+              if (q > 127.f) q = 127.f;
+              dst[e] = (uint8_t)(int8_t)q;
+            } else {
+              memcpy(dst + 2 * e, &hb, 2);
+            }
+          }
+        }
+    if (!zrow.alloc(512) || hipMemset(zrow.p, 0, 512) != hipSuccess ||
+        !wfrag32.alloc(f32.size()) || hipMemcpy(wfrag32.p, f32.data(), f32.size(), hipMemcpyHostToDevice) != hipSuccess) {
+      set_error("weight upload failed");
+      return false;
+    }
+  }
   if (!wfrag.alloc(frag.size()) || !wscale.alloc(ws.size() * 4) || !bias.alloc(bs.size() * 4)) return false;
   if (hipMemcpy(wfrag.p, frag.data(), frag.size(), hipMemcpyHostToDevice) != hipSuccess ||
       hipMemcpy(wscale.p, ws.data(), ws.size() * 4, hipMemcpyHostToDevice) != hipSuccess ||
@@ -1133,7 +1607,7 @@ bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* 
 static int conv_impl() {
   static const int impl = [] {
     const char* e = getenv("SCN_CONV_IMPL");
-    return (e && !strcmp(e, "rows")) ? 1 : 0;
+    return (e && !strcmp(e, "rows")) ? 1 : (e && !strcmp(e, "wg16")) ? 2 : (e && !strcmp(e, "reg32")) ? 3 : 0;
   }();
   return impl;
 }
@@ -1148,11 +1622,77 @@ static void launch_conv_rows(const ConvArgs& a, hipStream_t stream) {
   constexpr int SPK = CHUNKS >= 4 ? CHUNKS / 4 : 1;
   constexpr bool lds_ok = 2 * SPK * MT * 64 * 16 + kConvMaxKvol * 64 * NT * 4 <= 64 * 1024;
   const uint32_t blocks = 8 * ceil_div(ceil_div(a.n_bound, rows_per_block), 8);  // see xcd_tile()
-  if (conv_impl() == 0 && lds_ok && a.kvol <= kConvMaxKvol) {
+  if (conv_impl() != 1 && lds_ok && a.kvol <= kConvMaxKvol) {
     if constexpr (lds_ok)
       hipLaunchKernelGGL((k_conv_wg<EL, CHUNKS, MT, NT>), dim3(blocks), dim3(256), 0, stream, a);
   } else {
     hipLaunchKernelGGL((k_conv_rows<EL, CHUNKS, MT, NT>), dim3(blocks), dim3(256), 0, stream, a);
+  }
+}
+
+// rows per wave of the 32x32 kernel, in 32-row tiles (environment variable SCN_CONV_NT, default 1)
+static int conv32_nt() {
+  static const int nt = [] {
+    const char* e = getenv("SCN_CONV_NT");
+    return (e && atoi(e) == 2) ? 2 : 1;
+  }();
+  return nt;
+}
+
+template <int EL, int CHUNKS, int MT, int NT>
+static void launch_conv32(const ConvArgs& a, hipStream_t stream) {
+  constexpr uint32_t R = 128 * NT;
+  const uint32_t blocks = 8 * ceil_div(ceil_div(a.n_bound, R), 8);  // see xcd_tile()
+  hipLaunchKernelGGL((k_conv32<EL, CHUNKS, MT, NT>), dim3(blocks), dim3(256), 0, stream, a);
+}
+
+template <int EL, int CHUNKS, int MT, int WAVES>
+static void launch_conv_lds(const ConvArgs& a, hipStream_t stream) {
+  constexpr uint32_t R = 32 * WAVES;
+  const uint32_t blocks = 8 * ceil_div(ceil_div(a.n_bound, R), 8);  // see xcd_tile()
+  hipLaunchKernelGGL((k_conv_lds<EL, CHUNKS, MT, WAVES>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
+}
+
+// SCN_CONV_IMPL=reg32 selects the register-gather 32x32 kernel, SCN_CONV_WAVES=4 four-wave workgroups
+static int conv_lds_waves() {
+  static const int v = [] {
+    const char* e = getenv("SCN_CONV_WAVES");
+    return (e && atoi(e) == 4) ? 4 : 8;
+  }();
+  return v;
+}
+
+template <int EL, int CHUNKS>
+static bool dispatch_mt32(int mt, const ConvArgs& a, hipStream_t stream) {
+  if (conv_impl() == 3) {
+    const int nt = conv32_nt();
+    switch (mt * 10 + nt) {
+      case 11: launch_conv32<EL, CHUNKS, 1, 1>(a, stream); return true;
+      case 21: launch_conv32<EL, CHUNKS, 2, 1>(a, stream); return true;
+      case 41: launch_conv32<EL, CHUNKS, 4, 1>(a, stream); return true;
+      default: return false;
+    }
+  }
+  switch (mt * 10 + conv_lds_waves()) {
+    case 14: launch_conv_lds<EL, CHUNKS, 1, 4>(a, stream); return true;
+    case 18: launch_conv_lds<EL, CHUNKS, 1, 8>(a, stream); return true;
+    case 24: launch_conv_lds<EL, CHUNKS, 2, 4>(a, stream); return true;
+    case 28: launch_conv_lds<EL, CHUNKS, 2, 8>(a, stream); return true;
+    case 44: launch_conv_lds<EL, CHUNKS, 4, 4>(a, stream); return true;
+    case 48: launch_conv_lds<EL, CHUNKS, 4, 8>(a, stream); return true;
+    default: return false;
+  }
+}
+
+template <int EL>
+static bool dispatch_chunks32(int chunks, int mt, const ConvArgs& a, hipStream_t stream) {
+  switch (chunks) {
+    case 1: return dispatch_mt32<EL, 1>(mt, a, stream);
+    case 2: return dispatch_mt32<EL, 2>(mt, a, stream);
+    case 4: return dispatch_mt32<EL, 4>(mt, a, stream);
+    case 8: return dispatch_mt32<EL, 8>(mt, a, stream);
+    case 16: return dispatch_mt32<EL, 16>(mt, a, stream);
+    default: return false;
   }
 }
 
@@ -1210,6 +1750,7 @@ int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, cons
   a.n_out_dev = n_out_dev;
   a.n_bound = n_bound;
   a.wfrag = w.wfrag.as<uint4>();
+  a.zrow = w.zrow.as<char>();
   a.steps = w.steps;
   a.wscale = w.wscale.as<float>();
   a.bias = w.bias.as<float>();
@@ -1243,8 +1784,18 @@ int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, cons
     const char* dbg = getenv("SCN_CONV_DEBUG");
     a.debug = dbg ? atoi(dbg) : 0;
   }
-  bool ok = w.precision == SCN_PRECISION_INT8 ? dispatch_chunks<0>(w.chunks, w.mtiles, a, stream)
-                                               : dispatch_chunks<1>(w.chunks, w.mtiles, a, stream);
+  bool ok = false;
+  const int mt32 = w.mtiles32;
+  if (mt32 >= 1 && mt32 <= 4 && w.kvol <= kConvMaxKvol && (conv_impl() == 0 || conv_impl() == 3)) {
+    a.wfrag = w.wfrag32.as<uint4>();
+    ok = w.precision == SCN_PRECISION_INT8 ? dispatch_chunks32<0>(w.chunks, mt32, a, stream)
+                                           : dispatch_chunks32<1>(w.chunks, mt32, a, stream);
+  }
+  if (!ok) {
+    a.wfrag = w.wfrag.as<uint4>();
+    ok = w.precision == SCN_PRECISION_INT8 ? dispatch_chunks<0>(w.chunks, w.mtiles, a, stream)
+                                           : dispatch_chunks<1>(w.chunks, w.mtiles, a, stream);
+  }
   SCN_REQUIRE(ok, SCN_ERR_UNSUPPORTED, "conv: no kernel for Cin=%d Cout=%d (chunks %d, m-tiles %d)", w.cin, w.cout,
               w.chunks, w.mtiles);
   SCN_HIP(hipGetLastError());

@@ -81,6 +81,9 @@ struct ConvWeights {
   int steps = 0;    // MFMA K-steps = ceil(kvol * chunks / 4)
   uint32_t cin_pad = 0;  // padded input channels the kernel expects (elements)
   DevBuf wfrag;     // [steps][mtiles][64] x 16 bytes, MFMA A-operand order
+  int mtiles32 = 0, steps32 = 0;
+  DevBuf zrow;      // 512 bytes of zeros
+  DevBuf wfrag32;   // cout > 16: [steps32][mtiles32][64] x 16 bytes, A-operand order of the 32x32 MFMA
   DevBuf wscale;    // fp32 [cout_pad]: s_w[c] (int8) or 1
   DevBuf bias;      // fp32 [cout_pad]
   bool init(const uint16_t* w_fp16, const int shape[5], const float* ranges, const uint16_t* bias_fp16, int prec);
