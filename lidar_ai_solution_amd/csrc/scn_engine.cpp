@@ -724,6 +724,7 @@ static int allocate_runtime(scn_engine& e) {
   CoordSet& c0 = e.coords[0];
   memcpy(c0.grid, e.in_grid, 12);
   if (!c0.own_table.buf.p && !c0.own_table.alloc_for(c0.cap)) return SCN_ERR_HIP;
+  if (!c0.own_table.alloc_filter(c0.grid)) return SCN_ERR_HIP;
   // propagate grids and capacities through the strided rulebooks (they were created in order)
   for (auto& up : e.rulebooks) {
     RbSlot& s = *up;

@@ -103,6 +103,44 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t x, uint32_t* s
 }
 
 // --------------------------------------------------------------------------------------------
+// Workgroup-level aggregation of bitmap ORs.  Atomics on a bitmap shared by all XCDs are resolved
+// outside the XCD-local L2 and are slow; rows arrive in (nearly) sorted order, so the rows of one
+// workgroup hit few distinct words.  The ORs are first combined in a small LDS hash of
+// (word index -> bits) and each distinct word then costs one global atomic.
+// --------------------------------------------------------------------------------------------
+constexpr uint32_t kAggSlots = 2048;  // power of two
+constexpr uint32_t kAggEmpty = 0xFFFFFFFFu;
+
+__device__ __forceinline__ void agg_init(uint32_t* keys, uint32_t* vals) {
+  for (uint32_t i = threadIdx.x; i < kAggSlots; i += blockDim.x) {
+    keys[i] = kAggEmpty;
+    vals[i] = 0;
+  }
+  __syncthreads();
+}
+
+__device__ __forceinline__ void agg_or(uint32_t* keys, uint32_t* vals, uint32_t* bitmap, uint32_t word, uint32_t bits) {
+  uint32_t slot = (word * 2654435761u) >> (32 - 11);
+  for (int probe = 0; probe < 16; ++probe) {
+    const uint32_t prev = atomicCAS(&keys[slot], kAggEmpty, word);
+    if (prev == kAggEmpty || prev == word) {
+      atomicOr(&vals[slot], bits);
+      return;
+    }
+    slot = (slot + 1) & (kAggSlots - 1);
+  }
+  atomicOr(&bitmap[word], bits);  // crowded table: straight to memory
+}
+
+__device__ __forceinline__ void agg_flush(const uint32_t* keys, const uint32_t* vals, uint32_t* bitmap) {
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < kAggSlots; i += blockDim.x) {
+    const uint32_t w = keys[i];
+    if (w != kAggEmpty) atomicOr(&bitmap[w], vals[i]);
+  }
+}
+
+// --------------------------------------------------------------------------------------------
 // fill
 // --------------------------------------------------------------------------------------------
 __global__ void k_fill_u32(uint32_t* __restrict__ p, uint32_t value, size_t count) {
@@ -135,17 +173,25 @@ __device__ __forceinline__ bool coord_key(const int4 c, const Int3 g, uint32_t* 
   return true;
 }
 
-__global__ void k_hash_insert(uint64_t* slots, uint32_t mask, const int4* __restrict__ coords, uint32_t n_bound,
-                              const uint32_t* n_dev, Int3 grid, uint32_t* n_eff_out) {
+// filter (nullable): occupancy bitmap of the grid, set for every inserted coordinate; lookups test it
+// before probing the table (most neighbour lookups of a sparse tensor miss).
+__global__ __launch_bounds__(256) void k_hash_insert(uint64_t* slots, uint32_t mask, const int4* __restrict__ coords,
+                                                     uint32_t n_bound, const uint32_t* n_dev, Int3 grid,
+                                                     uint32_t* n_eff_out, uint32_t* filter) {
+  __shared__ uint32_t akeys[kAggSlots], avals[kAggSlots];
   const uint32_t n = eff_n(n_dev, n_bound);
   const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
   if (r == 0 && n_eff_out) {
     n_eff_out[0] = n;
     n_eff_out[1] = n;
   }
-  if (r >= n) return;
+  if (filter) agg_init(akeys, avals);
   uint32_t key;
-  if (coord_key(coords[r], grid, &key)) table_insert(slots, mask, key, r);
+  if (r < n && coord_key(coords[r], grid, &key)) {
+    table_insert(slots, mask, key, r);
+    if (filter) agg_or(akeys, avals, filter, key >> 5, 1u << (key & 31));
+  }
+  if (filter) agg_flush(akeys, avals, filter);
 }
 
 __global__ void k_hash_query(const uint64_t* __restrict__ slots, uint32_t mask, const int4* __restrict__ coords,
@@ -168,6 +214,20 @@ bool CoordTable::alloc_for(uint32_t max_rows) {
   return buf.alloc(cap * sizeof(uint64_t));
 }
 
+// Occupancy filter of the whole grid, one bit per cell; skipped (lookups then go straight to the
+// table) for grids above 2^29 cells = 64 MB of bitmap.
+bool CoordTable::alloc_filter(const int grid[3]) {
+  const uint64_t cells = (uint64_t)grid[0] * (uint64_t)grid[1] * (uint64_t)grid[2];
+  if (cells == 0 || cells > (1ull << 29)) {
+    filter_words = 0;
+    return true;
+  }
+  const size_t words = (size_t)((cells + 31) / 32 + 3) & ~(size_t)3;
+  if (words > filter.bytes / 4 && !filter.alloc(words * 4)) return false;
+  filter_words = words;
+  return true;
+}
+
 static bool grid_fits_u32(const int g[3]) {
   if (g[0] <= 0 || g[1] <= 0 || g[2] <= 0) return false;
   const uint64_t vol = (uint64_t)g[0] * (uint64_t)g[1] * (uint64_t)g[2];
@@ -183,10 +243,14 @@ int hash_build(const CoordTable& t, const int32_t* idx, uint32_t n, const uint32
   const_cast<CoordTable&>(t).mask = (uint32_t)(hash_capacity_for(n) - 1);
   int rc = fill_u32(t.slots(), 0xFFFFFFFFu, ((size_t)t.mask + 1) * 2, stream);
   if (rc) return rc;
+  if (t.filter_words) {
+    rc = fill_u32(t.filter.p, 0u, t.filter_words, stream);
+    if (rc) return rc;
+  }
   Int3 g{{grid[0], grid[1], grid[2]}};
   const uint32_t blocks = n ? ceil_div(n, 256) : 1;
   hipLaunchKernelGGL(k_hash_insert, dim3(blocks), dim3(256), 0, stream, t.slots(), t.mask,
-                     (const int4*)idx, n, n_dev, g, n_eff_out);
+                     (const int4*)idx, n, n_dev, g, n_eff_out, t.filter_words ? t.filter.as<uint32_t>() : nullptr);
   SCN_HIP(hipGetLastError());
   return SCN_OK;
 }
@@ -317,6 +381,7 @@ __device__ __forceinline__ int32_t coord_row(const CoordLookup& lk, uint32_t key
     const uint32_t r = lk.prefix[key >> 5] + __popc(w & ((1u << b) - 1u));
     return r < lk.rank_cap ? (int32_t)r : -1;
   }
+  if (lk.filter && !((lk.filter[key >> 5] >> (key & 31)) & 1u)) return -1;
   return table_lookup(lk.slots, lk.mask, key);
 }
 
@@ -359,39 +424,49 @@ __global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_
 
 // Marks every output cell reached by an input row through some kernel offset.  One thread per
 // input row; per axis the (at most K) reachable output coordinates are found first, then their
-// combinations are marked.  The bit is tested before the atomic so that cells reached by several
-// inputs cost one atomic, not one per input.
+// combinations are marked -- the bits of one output line that fall into the same word in one
+// operation, through the workgroup's LDS aggregation (see agg_or).
 __global__ __launch_bounds__(256) void k_mark_outputs(const int4* __restrict__ in_coords, const uint32_t* n_dev,
                                                       uint32_t n_bound, GeomDev g, uint32_t* bitmap) {
+  __shared__ uint32_t akeys[kAggSlots], avals[kAggSlots];
+  agg_init(akeys, avals);
   const uint32_t n = eff_n(n_dev, n_bound);
   const uint32_t r = blockIdx.x * 256 + threadIdx.x;
-  if (r >= n) return;
-  const int4 c = in_coords[r];
-  if (c.x != 0 || c.y < 0 || c.y >= g.gi[0] || c.z < 0 || c.z >= g.gi[1] || c.w < 0 || c.w >= g.gi[2]) return;
-  const int cc[3] = {c.y, c.z, c.w};
-  constexpr int kMaxK = 8;  // per-axis kernel sizes above this fall back to the generic loop bound
-  int o[3][kMaxK];
-  int cnt[3] = {0, 0, 0};
+  int4 c = make_int4(-1, 0, 0, 0);
+  if (r < n) c = in_coords[r];
+  if (c.x == 0 && c.y >= 0 && c.y < g.gi[0] && c.z >= 0 && c.z < g.gi[1] && c.w >= 0 && c.w < g.gi[2]) {
+    const int cc[3] = {c.y, c.z, c.w};
+    constexpr int kMaxK = 8;  // per-axis kernel sizes are limited to 8 by the host checks
+    int o[3][kMaxK];
+    int cnt[3] = {0, 0, 0};
 #pragma unroll
-  for (int a = 0; a < 3; ++a) {
-    const int ks = g.ks[a] < kMaxK ? g.ks[a] : kMaxK;
-    for (int k = 0; k < ks; ++k) {
-      const int t = cc[a] + g.pd[a] - k * g.dl[a];
-      if (t < 0) continue;
-      const int q = t / g.st[a];
-      if (q * g.st[a] != t || q >= g.go[a]) continue;
-      o[a][cnt[a]++] = q;
-    }
-  }
-  for (int a0 = 0; a0 < cnt[0]; ++a0)
-    for (int a1 = 0; a1 < cnt[1]; ++a1) {
-      const uint32_t line = ((uint32_t)o[0][a0] * (uint32_t)g.go[1] + (uint32_t)o[1][a1]) * (uint32_t)g.go[2];
-      for (int a2 = 0; a2 < cnt[2]; ++a2) {
-        const uint32_t key = line + (uint32_t)o[2][a2];
-        const uint32_t bit = 1u << (key & 31);
-        if (!(bitmap[key >> 5] & bit)) atomicOr(&bitmap[key >> 5], bit);
+    for (int a = 0; a < 3; ++a) {
+      const int ks = g.ks[a] < kMaxK ? g.ks[a] : kMaxK;
+      for (int k = 0; k < ks; ++k) {
+        const int t = cc[a] + g.pd[a] - k * g.dl[a];
+        if (t < 0) continue;
+        const int q = t / g.st[a];
+        if (q * g.st[a] != t || q >= g.go[a]) continue;
+        o[a][cnt[a]++] = q;
       }
     }
+    for (int a0 = 0; a0 < cnt[0]; ++a0)
+      for (int a1 = 0; a1 < cnt[1]; ++a1) {
+        const uint32_t line = ((uint32_t)o[0][a0] * (uint32_t)g.go[1] + (uint32_t)o[1][a1]) * (uint32_t)g.go[2];
+        uint32_t word = kAggEmpty, bits = 0;
+        for (int a2 = 0; a2 < cnt[2]; ++a2) {
+          const uint32_t key = line + (uint32_t)o[2][a2];
+          if ((key >> 5) != word) {
+            if (bits) agg_or(akeys, avals, bitmap, word, bits);
+            word = key >> 5;
+            bits = 0;
+          }
+          bits |= 1u << (key & 31);
+        }
+        if (bits) agg_or(akeys, avals, bitmap, word, bits);
+      }
+  }
+  agg_flush(akeys, avals, bitmap);
 }
 
 bool Rulebook::init(uint32_t max_in_, uint32_t max_out_, int kvol) {
@@ -443,6 +518,7 @@ CoordLookup CoordTable::lookup() const {
   CoordLookup lk;
   lk.slots = slots();
   lk.mask = mask;
+  lk.filter = filter_words ? filter.as<uint32_t>() : nullptr;
   return lk;
 }
 
@@ -479,6 +555,7 @@ int Rulebook::build_subm(const int32_t* idx, uint32_t n, const uint32_t* n_dev, 
   } else {
     rc = reserve_subm(true);
     if (rc) return rc;
+    if (!own_in_table.alloc_filter(grid)) return SCN_ERR_HIP;
     rc = hash_build(own_in_table, idx, n, n_dev, grid, nullptr, stream);
     if (rc) return rc;
     in_lookup = own_in_table.lookup();
@@ -551,6 +628,7 @@ int Rulebook::build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev
   if (shared_lookup) {
     in_lookup = *shared_lookup;
   } else {
+    if (!own_in_table.alloc_filter(grid)) return SCN_ERR_HIP;
     rc = hash_build(own_in_table, idx, n, n_dev, grid, nullptr, stream);
     if (rc) return rc;
     in_lookup = own_in_table.lookup();
@@ -1285,32 +1363,38 @@ __global__ __launch_bounds__(256, 2) void k_conv32(const ConvArgs a) {
 // What bounds the register-gather kernels above is the vector-memory path, not the matrix cores: a
 // gather in MFMA operand order (32 rows x 2 lanes x 16 B) costs ~97 cycles of a CU's texture pipe per
 // instruction, one whose 8 adjacent lanes read one row's 128 contiguous bytes ~35 (both measured,
-// L2-resident table).  So rows are gathered in the memory-friendly order, straight into LDS
-// (global_load_lds_dwordx4: no registers, no masking -- lanes without a neighbour read a row of zeros),
-// two iterations ahead, and the MFMA B operand is read back from LDS.  Hardware places lane l's 16 bytes
-// at base + 16 l, so the bank-conflict-free read order is obtained by permuting which chunk of its row
-// a lane fetches: position p of a row holds chunk p ^ swz(row).
+// cache-resident table).  So everything that comes from global memory -- gathered rows, weight slabs,
+// neighbour indices -- is loaded in memory-friendly order straight into LDS (global_load_lds: no
+// registers, no masking; lanes without a neighbour read a row of zeros) and the MFMA operands are read
+// back from LDS.  With no staging registers the kernel fits 128 VGPRs, so two 8-wave workgroups (four
+// waves per SIMD, 512 output rows) share a CU and hide each other's latencies.
+// Hardware places lane l's bytes at base + 16 l, so the bank-conflict-free read order of the B operand is
+// obtained by permuting which chunk of its row a lane fetches: position p of a row holds chunk p ^ swz(row).
 //   iteration     = 4 K-steps = 4 KB of gathered rows per wave (32 rows x 8 chunks, or G = 8 / SEG
 //                   kernel offsets of SEG-chunk rows) and a weight slab of 4 * MT fragments
-//   weight slabs  = global -> registers -> LDS (triple buffered), A fragments of iteration i+1 are read
-//                   from LDS during iteration i
-//   per iteration = one barrier; each wave consumes only rows it gathered itself, so gathers need a
-//                   wait on the wave's own memory counter, not a barrier
+//   LDS           = 2 weight slabs (iteration i, i+1), one 4 KB stage of gathered rows per wave, and a
+//                   4-deep ring of neighbour indices per wave (they always miss the caches)
+//   per iteration = one barrier for the slab; a wave consumes only rows and indices it fetched itself,
+//                   so those need a wait on the wave's own memory counter only
+// The memory counter retires loads in order, so "at most N outstanding" names exactly which older load
+// has landed.  Issue order per iteration i: slab S(i+1), indices I(i+4), gathers G(i+1).
 template <int EL, int CHUNKS, int MT, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void k_conv_lds(const ConvArgs a) {
+__global__ __launch_bounds__(64 * WAVES, 4) void k_conv_lds(const ConvArgs a) {
   using Acc = typename Mma32<EL>::Acc;
   using Acc4 = typename Mma32<EL>::Acc4;
   constexpr int THREADS = 64 * WAVES;
   constexpr int SEG = CHUNKS < 8 ? CHUNKS : 8;   // chunks gathered per row and iteration
   constexpr int IPO = CHUNKS / SEG;              // iterations per kernel offset (rows wider than 128 B)
   constexpr int G = 8 / SEG;                     // kernel offsets per iteration
-  constexpr int RP = 8 / SEG;                    // rows per 128 bytes of a gathered stage
+  constexpr int RP = 8 / SEG;                    // rows per 128 bytes of the gathered stage
   constexpr int SLAB = 4 * MT * 64;              // 16-byte weight fragments per iteration
-  constexpr int WPT = (SLAB + THREADS - 1) / THREADS;
+  static_assert(SLAB % THREADS == 0, "every wave must issue the same number of slab loads");
+  constexpr int WPT = SLAB / THREADS;            // slab loads per wave and iteration
+  constexpr int IDXI = G >= 2 ? G / 2 : 1;       // index loads per wave and iteration (64 entries each)
   constexpr int R = 32 * WAVES;                  // output rows per workgroup
-  __shared__ v4i lds[3][SLAB];
-  __shared__ v4i ring[2][WAVES][256];            // gathered rows: two stages of 4 KB per wave
-  __shared__ int32_t lidx[kConvMaxKvol * R];
+  __shared__ v4i lds[2][SLAB];
+  __shared__ v4i ring[WAVES][256];
+  __shared__ int32_t iring[4][WAVES][64 * IDXI];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, lh = lane >> 5;
@@ -1318,56 +1402,12 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_lds(const ConvArgs a) {
   uint32_t tile;
   if (!xcd_tile(n, R, &tile)) return;
   const uint32_t row0 = (tile * WAVES + wave) * 32;
-  {
-    const uint32_t tile_row0 = tile * R;
-    const int total = a.kvol * R;
-    for (int base = 0; base < total; base += THREADS * 8) {
-      int32_t tmp[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int f = base + j * THREADS + tid;
-        const int k = f / R, r = f - k * R;
-        const bool v = f < total && tile_row0 + r < n;
-        tmp[j] = v ? a.nbr[(size_t)k * a.nbr_ld + tile_row0 + r] : -1;
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int f = base + j * THREADS + tid;
-        if (f < total) lidx[f] = tmp[j];
-      }
-    }
-  }
-  __syncthreads();
   const int iters = IPO > 1 ? a.kvol * IPO : (a.kvol + G - 1) / G;
-  const int last = iters - 1;
   const char* __restrict__ xb = a.x;
   const char* __restrict__ zrow = a.zrow;
   const v4i* __restrict__ wsrc = reinterpret_cast<const v4i*>(a.wfrag);
   const uint32_t ldb = a.x_ld_bytes;
-
-  // this lane's four gather slots: element e = 64 q + lane of the stage's [G][32 rows][SEG] array
-  int g_row[4], g_off[4], g_chunk[4];
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const int e = q * 64 + lane;
-    const int row = (e / SEG) % 32, c = e % SEG;
-    g_off[q] = e / (32 * SEG);
-    g_row[q] = row;
-    g_chunk[q] = c ^ ((row / RP) % SEG);
-  }
-  // this lane's B-operand read positions (16-byte units inside a stage) for the 4 K-steps
-  int b_pos[4];
-#pragma unroll
-  for (int ss = 0; ss < 4; ++ss) {
-    if (SEG >= 2) {
-      constexpr int SPO = SEG >= 2 ? SEG / 2 : 1;
-      const int g = ss / SPO, cl = 2 * (ss % SPO) + lh;
-      b_pos[ss] = (g * 32 + ln) * SEG + (cl ^ ((ln / RP) % SEG));
-    } else {
-      b_pos[ss] = (2 * ss + lh) * 32 + ln;
-    }
-  }
-  const int32_t* __restrict__ my_idx = lidx + wave * 32;
+  const int32_t* __restrict__ minus1 = reinterpret_cast<const int32_t*>(a.zrow + 512);  // words of -1
 
   Acc acc[MT];
 #pragma unroll
@@ -1375,118 +1415,173 @@ __global__ __launch_bounds__(64 * WAVES) void k_conv_lds(const ConvArgs a) {
 #pragma unroll
     for (int j = 0; j < 16; ++j) acc[t][j] = 0;
 
-// neighbour rows of this lane's four gather slots of iteration IT (-1: none)
-#define SCN_GATHER_IDX(IT, GI)                                                                  \
-  {                                                                                             \
-    _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                             \
-      const int k_ = IPO > 1 ? (IT) / IPO : (IT) * G + g_off[q];                                \
-      const bool kv_ = (IT) < iters && k_ < a.kvol;                                             \
-      GI[q] = my_idx[(kv_ ? k_ : 0) * R + g_row[q]];                                            \
-    }                                                                                           \
-  }
-// gathers of iteration IT into ring stage STG: lanes whose slot has no neighbour (or lies beyond the
-// kernel volume / the iteration count) read the row of zeros
-#define SCN_GATHER(IT, STG, GI)                                                                 \
-  {                                                                                             \
-    _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                             \
-      const int k_ = IPO > 1 ? (IT) / IPO : (IT) * G + g_off[q];                                \
-      const bool kv_ = (IT) < iters && k_ < a.kvol;                                             \
-      const int cg_ = (IPO > 1 ? ((IT) % IPO) * 8 : 0) + g_chunk[q];                            \
-      const char* p_ = (kv_ && GI[q] >= 0) ? xb + (size_t)(uint32_t)GI[q] * ldb + cg_ * 16 : zrow + cg_ * 16; \
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)p_,       \
-                                       (__attribute__((address_space(3))) void*)&ring[STG][wave][q * 64], 16, 0, 0); \
-    }                                                                                           \
-  }
-#define SCN_LOAD_SLAB(IT, W)                                                                    \
-  {                                                                                             \
-    const int it_ = (IT) < last ? (IT) : last;                                                  \
-    _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                                           \
-      const int f_ = tid + j * THREADS;                                                         \
-      W[j] = wsrc[(size_t)it_ * SLAB + ((SLAB % THREADS == 0 || f_ < SLAB) ? f_ : 0)];          \
-    }                                                                                           \
-  }
-#define SCN_STORE_SLAB(BUF, W)                                                                  \
-  {                                                                                             \
-    _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                                           \
-      const int f_ = tid + j * THREADS;                                                         \
-      if (SLAB % THREADS == 0 || f_ < SLAB) lds[BUF][f_] = W[j];                                \
-    }                                                                                           \
-  }
-// Waits are explicit in the loop: the wave's memory counter retires loads in order, so "at most N
-// outstanding" identifies exactly which older load has landed.  Issue order per iteration IT:
-//   slab load S(IT) (WPT loads, top)  ->  gathers G(IT+2) (4 loads, after K-step 0)
+  typedef const __attribute__((address_space(1))) void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
 #define SCN_WAIT_VM(N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory")
-// Barrier that waits for the wave's LDS traffic except the KEEP newest operations (LDS completes in
-// order).  __syncthreads() would also drain the memory counter, i.e. every gather in flight.
-#define SCN_LDS_BARRIER(KEEP) asm volatile("s_waitcnt lgkmcnt(%0)\n\ts_barrier" ::"n"(KEEP) : "memory")
-// one iteration; STG = ring stage of its gathered rows (IT % 2), already read into BC
-#define SCN_ITER(IT, STG, BC, BN, WC, WN)                                                       \
+// LDS reads of what global_load_lds wrote are written in assembly: the compiler orders a visible LDS read
+// after EVERY outstanding global_load_lds (vmcnt(0)), which would drain the loads issued for the next
+// iterations.  The waits that are really needed are the explicit ones below.
+// weight slab of iteration IT -> LDS buffer IT % 2 (iterations past the end re-load the last slab)
+#define SCN_SLAB(IT)                                                                            \
   {                                                                                             \
-    SCN_LOAD_SLAB((IT) + 3, WN);                                                                \
-    int32_t gi[4];                                                                              \
-    SCN_GATHER_IDX((IT) + 2, gi);                                                               \
-    const int nxt_ = cur == 2 ? 0 : cur + 1;                                                    \
-    const int nn_ = nxt_ == 2 ? 0 : nxt_ + 1;                                                   \
-    SCN_WAIT_VM(WPT + 4); /* S(IT-1) landed; younger: G(IT+1), S(IT) */                         \
-    SCN_STORE_SLAB(nn_, WC);                                                                    \
-    __builtin_amdgcn_sched_barrier(0);                                                          \
-    const v4i* la = &lds[nxt_][0] + lane;                                                       \
-    _Pragma("unroll") for (int ss = 0; ss < 4; ++ss) {                                          \
-      _Pragma("unroll") for (int t = 0; t < MT; ++t)                                            \
-        acc[t] = Mma32<EL>::run(af[ss][t], BC[ss], acc[t]);                                     \
-      _Pragma("unroll") for (int t = 0; t < MT; ++t) af[ss][t] = la[(ss * MT + t) * 64];        \
-      /* stage STG was read into BC during the previous iteration: free for the gathers of IT+2 */ \
-      if (ss == 0) SCN_GATHER((IT) + 2, STG, gi);                                               \
-      if (ss == 1) {                                                                            \
-        SCN_WAIT_VM(WPT + 4); /* G(IT+1) landed; younger: S(IT), G(IT+2) */                     \
-        _Pragma("unroll") for (int s2 = 0; s2 < 4; ++s2) BN[s2] = ring[(STG) ^ 1][wave][b_pos[s2]]; \
-      }                                                                                         \
-      __builtin_amdgcn_sched_barrier(0);                                                        \
+    const int it_ = (IT) < iters ? (IT) : iters - 1;                                            \
+    _Pragma("unroll") for (int j = 0; j < WPT; ++j)                                             \
+      __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + (size_t)it_ * SLAB + j * THREADS + tid), \
+                                       (lptr_t)&lds[(IT) & 1][j * THREADS + wave * 64], 16, 0, 0); \
+  }
+// neighbour rows of iteration IT -> index ring stage IT % 4: entry e = 64 q + lane is kernel offset
+// e / 32 of the iteration, tile row e % 32; slots outside the volume or beyond row n read -1
+#define SCN_INDEX(IT)                                                                           \
+  {                                                                                             \
+    _Pragma("unroll") for (int q = 0; q < IDXI; ++q) {                                          \
+      const int e_ = q * 64 + lane;                                                             \
+      const int k_ = IPO > 1 ? (IT) / IPO + e_ / 32 : (IT) * G + e_ / 32;                       \
+      const uint32_t r_ = row0 + (e_ & 31);                                                     \
+      const bool ok_ = (IT) < iters && k_ < a.kvol && r_ < n;                                   \
+      const int32_t* p_ = ok_ ? a.nbr + (size_t)k_ * a.nbr_ld + r_ : minus1 + lane;             \
+      __builtin_amdgcn_global_load_lds((gptr_t)p_, (lptr_t)&iring[(IT) & 3][wave][q * 64], 4, 0, 0); \
     }                                                                                           \
-    SCN_LDS_BARRIER(MT); /* all but the last MT fragment refills */                             \
-    cur = nxt_;                                                                                 \
+  }
+// gathers of iteration IT (neighbour rows GI[4] of this lane's slots) into the wave's stage; element
+// e = 64 q + lane of its [G][32 rows][SEG] array
+#define SCN_GATHER(IT, GI)                                                                      \
+  {                                                                                             \
+    _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                             \
+      const int e_ = q * 64 + lane;                                                             \
+      const int row_ = (e_ / SEG) % 32;                                                         \
+      const int cg_ = (IPO > 1 ? ((IT) % IPO) * 8 : 0) + ((e_ % SEG) ^ ((row_ / RP) % SEG));    \
+      const char* p_ = GI[q] >= 0 ? xb + (size_t)(uint32_t)GI[q] * ldb + cg_ * 16 : zrow + cg_ * 16; \
+      __builtin_amdgcn_global_load_lds((gptr_t)p_, (lptr_t)&ring[wave][q * 64], 16, 0, 0);      \
+    }                                                                                           \
+  }
+// this lane's four index slots of ring stage STG -> GI[4], waited for.  Slot q of lane l is entry
+// e / SEG of the stage (e = 64 q + l), i.e. a fixed stride of 64 / SEG entries between slots.
+#define SCN_READ_INDEX(STG, GI)                                                                 \
+  {                                                                                             \
+    const uint32_t base_ = iring_addr + (uint32_t)(STG) * (WAVES * 64 * IDXI * 4);              \
+    asm volatile("ds_read_b32 %0, %4\n\tds_read_b32 %1, %4 offset:%5\n\tds_read_b32 %2, %4 offset:%6\n\t" \
+                 "ds_read_b32 %3, %4 offset:%7\n\ts_waitcnt lgkmcnt(0)"                         \
+                 : "=&v"(GI[0]), "=&v"(GI[1]), "=&v"(GI[2]), "=&v"(GI[3])                       \
+                 : "v"(base_), "n"(256 / SEG), "n"(2 * 256 / SEG), "n"(3 * 256 / SEG)           \
+                 : "memory");                                                                   \
+  }
+// A fragments of K-step SS from the slab at LDS byte address LA (+ lane * 16 already included)
+#define SCN_READ_A(SS, LA, AF)                                                                  \
+  {                                                                                             \
+    if constexpr (MT == 4)                                                                      \
+      asm volatile("ds_read_b128 %0, %4 offset:%5\n\tds_read_b128 %1, %4 offset:%6\n\t"         \
+                   "ds_read_b128 %2, %4 offset:%7\n\tds_read_b128 %3, %4 offset:%8"             \
+                   : "=&v"(AF[0]), "=&v"(AF[1]), "=&v"(AF[2]), "=&v"(AF[3])                     \
+                   : "v"(LA), "n"(((SS) * 4 + 0) * 1024), "n"(((SS) * 4 + 1) * 1024),           \
+                     "n"(((SS) * 4 + 2) * 1024), "n"(((SS) * 4 + 3) * 1024)                     \
+                   : "memory");                                                                 \
+    else if constexpr (MT == 2)                                                                 \
+      asm volatile("ds_read_b128 %0, %2 offset:%3\n\tds_read_b128 %1, %2 offset:%4"             \
+                   : "=&v"(AF[0]), "=&v"(AF[1])                                                 \
+                   : "v"(LA), "n"(((SS) * 2 + 0) * 1024), "n"(((SS) * 2 + 1) * 1024)            \
+                   : "memory");                                                                 \
+    else                                                                                        \
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(AF[0]) : "v"(LA), "n"((SS) * 1024) : "memory"); \
+  }
+// wait until at most KEEP LDS operations are outstanding; AF is named as in/out so that its MFMAs stay below
+#define SCN_WAIT_A(KEEP, AF)                                                                    \
+  {                                                                                             \
+    if constexpr (MT == 4)                                                                      \
+      asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(AF[0]), "+v"(AF[1]), "+v"(AF[2]), "+v"(AF[3]) : "n"(KEEP) : "memory"); \
+    else if constexpr (MT == 2)                                                                 \
+      asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(AF[0]), "+v"(AF[1]) : "n"(KEEP) : "memory");  \
+    else                                                                                        \
+      asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(AF[0]) : "n"(KEEP) : "memory");               \
   }
 
-  v4i wA[WPT], wB[WPT];
-  v4i af[4][MT];
-  v4i bfA[4], bfB[4];
-  int cur = 0;
+  const uint32_t ring_addr = (uint32_t)(uintptr_t)(lptr_t)&ring[wave][0];
+  const uint32_t iring_addr = (uint32_t)(uintptr_t)(lptr_t)&iring[0][wave][0] + (uint32_t)(lane / SEG) * 4;
+  const uint32_t lds_a_addr = (uint32_t)(uintptr_t)(lptr_t)&lds[0][lane];
+  // B-operand read address of K-step ss inside the wave's stage: row ln, chunk 2 ss' + lh at its swizzled
+  // position.  Recomputed per iteration from two values (registers are what limits occupancy here).
+  const uint32_t b_base = ring_addr + (uint32_t)(SEG >= 2 ? ln * SEG : lh * 32 + ln) * 16;
+  const uint32_t b_swz = SEG >= 2 ? (uint32_t)(lh ^ ((ln / RP) % SEG)) : 0u;
+#define SCN_B_ADDR(SS, BB, SW)                                                                  \
+  (SEG >= 2 ? (BB) + (uint32_t)((((SS) / (SEG / 2 > 0 ? SEG / 2 : 1)) * 32 * SEG) +             \
+                                ((2 * ((SS) % (SEG / 2 > 0 ? SEG / 2 : 1))) ^ (SW))) * 16       \
+            : (BB) + (uint32_t)(2 * (SS) * 32) * 16)
+
+  // prologue: indices of iterations 0..3, slab 0, then the gathers of iteration 0
+  SCN_INDEX(0);
+  SCN_INDEX(1);
+  SCN_INDEX(2);
+  SCN_INDEX(3);
+  SCN_SLAB(0);
+  SCN_WAIT_VM(0);
   {
-    int32_t g0[4], g1[4];
-    SCN_GATHER_IDX(0, g0);
-    SCN_GATHER_IDX(1, g1);
-    SCN_LOAD_SLAB(0, wA);
-    SCN_LOAD_SLAB(1, wB);
-    SCN_GATHER(0, 0, g0);
-    SCN_WAIT_VM(4);
-    SCN_STORE_SLAB(0, wA);
-    SCN_STORE_SLAB(1, wB);
-    __builtin_amdgcn_sched_barrier(0);
-    SCN_LOAD_SLAB(2, wB);
-    SCN_GATHER(1, 1, g1);
+    int32_t gi[4];
+    SCN_READ_INDEX(0, gi);
+    SCN_GATHER(0, gi);
   }
-  SCN_LDS_BARRIER(0);
+  asm volatile("s_barrier" ::: "memory");
+
+  for (int it = 0; it < iters; ++it) {
+    SCN_SLAB(it + 1);
+    SCN_INDEX(it + 4);
+    SCN_WAIT_VM(WPT + IDXI);  // G(it), I(it+1) and everything older have landed
+    v4i bf[4];
+    int32_t gi[4];
+    {
+      uint32_t bb = b_base, sw = b_swz;
+      asm volatile("" : "+v"(bb), "+v"(sw));  // keeps the four addresses out of loop-carried registers
+      asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\tds_read_b128 %3, %7"
+                   : "=&v"(bf[0]), "=&v"(bf[1]), "=&v"(bf[2]), "=&v"(bf[3])
+                   : "v"(SCN_B_ADDR(0, bb, sw)), "v"(SCN_B_ADDR(1, bb, sw)), "v"(SCN_B_ADDR(2, bb, sw)),
+                     "v"(SCN_B_ADDR(3, bb, sw))
+                   : "memory");
+    }
+    // waits for the index reads and, LDS returning in order, for bf[]: the stage may be overwritten
+    SCN_READ_INDEX((it + 1) & 3, gi);
+    SCN_GATHER(it + 1, gi);
+    const uint32_t la = lds_a_addr + (uint32_t)(it & 1) * (SLAB * 16);
+    if constexpr (MT >= 4) {
+      // 64 accumulator registers leave room for one set of fragments under the 128-register budget of
+      // four waves per SIMD (a spill would also put scratch loads into the memory counter and break the
+      // counts above); the other three waves of the SIMD cover the LDS latency instead
+      v4i af[MT];
 #pragma unroll
-  for (int ss = 0; ss < 4; ++ss)
+      for (int ss = 0; ss < 4; ++ss) {
+        SCN_READ_A(ss, la, af);
+        SCN_WAIT_A(0, af);
 #pragma unroll
-    for (int t = 0; t < MT; ++t) af[ss][t] = lds[0][(ss * MT + t) * 64 + lane];
-  SCN_WAIT_VM(WPT + 4);  // G(0) landed; younger: S(2), G(1)
+        for (int t = 0; t < MT; ++t) acc[t] = Mma32<EL>::run(af[t], bf[ss], acc[t]);
+      }
+    } else {
+      v4i afA[MT], afB[MT];
+      SCN_READ_A(0, la, afA);
+      SCN_READ_A(1, la, afB);
+      SCN_WAIT_A(MT, afA);
 #pragma unroll
-  for (int ss = 0; ss < 4; ++ss) bfA[ss] = ring[0][wave][b_pos[ss]];
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  int it = 0;
-  for (; it + 1 < iters; it += 2) {
-    SCN_ITER(it, 0, bfA, bfB, wB, wA);
-    SCN_ITER(it + 1, 1, bfB, bfA, wA, wB);
+      for (int t = 0; t < MT; ++t) acc[t] = Mma32<EL>::run(afA[t], bf[0], acc[t]);
+      SCN_READ_A(2, la, afA);
+      SCN_WAIT_A(MT, afB);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = Mma32<EL>::run(afB[t], bf[1], acc[t]);
+      SCN_READ_A(3, la, afB);
+      SCN_WAIT_A(MT, afA);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = Mma32<EL>::run(afA[t], bf[2], acc[t]);
+      SCN_WAIT_A(0, afB);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = Mma32<EL>::run(afB[t], bf[3], acc[t]);
+    }
+    SCN_WAIT_VM(4);  // this wave's part of S(it+1) has landed (younger: G(it+1))
+    // every wave has read slab it (its fragments are in registers) and written its part of slab it+1
+    asm volatile("s_barrier" ::: "memory");
   }
-  if (it < iters) SCN_ITER(it, 0, bfA, bfB, wB, wA);
+#undef SCN_READ_INDEX
+#undef SCN_B_ADDR
+#undef SCN_READ_A
+#undef SCN_WAIT_A
 #undef SCN_WAIT_VM
-#undef SCN_GATHER_IDX
-#undef SCN_LDS_BARRIER
+#undef SCN_SLAB
+#undef SCN_INDEX
 #undef SCN_GATHER
-#undef SCN_LOAD_SLAB
-#undef SCN_STORE_SLAB
-#undef SCN_ITER
   const uint32_t row = row0 + ln;
   if (row >= n) return;
   const int cout_pad = (a.cout + 15) & ~15;
@@ -1586,7 +1681,8 @@ bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* 
             }
           }
         }
-    if (!zrow.alloc(512) || hipMemset(zrow.p, 0, 512) != hipSuccess ||
+    if (!zrow.alloc(768) || hipMemset(zrow.p, 0, 512) != hipSuccess ||
+        hipMemset(zrow.as<char>() + 512, 0xFF, 256) != hipSuccess ||  // 64 words of -1 ("no neighbour")
         !wfrag32.alloc(f32.size()) || hipMemcpy(wfrag32.p, f32.data(), f32.size(), hipMemcpyHostToDevice) != hipSuccess) {
       set_error("weight upload failed");
       return false;
@@ -1653,15 +1749,7 @@ static void launch_conv_lds(const ConvArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL((k_conv_lds<EL, CHUNKS, MT, WAVES>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
 }
 
-// SCN_CONV_IMPL=reg32 selects the register-gather 32x32 kernel, SCN_CONV_WAVES=4 four-wave workgroups
-static int conv_lds_waves() {
-  static const int v = [] {
-    const char* e = getenv("SCN_CONV_WAVES");
-    return (e && atoi(e) == 4) ? 4 : 8;
-  }();
-  return v;
-}
-
+// SCN_CONV_IMPL=reg32 selects the register-gather 32x32 kernel
 template <int EL, int CHUNKS>
 static bool dispatch_mt32(int mt, const ConvArgs& a, hipStream_t stream) {
   if (conv_impl() == 3) {
@@ -1673,13 +1761,10 @@ static bool dispatch_mt32(int mt, const ConvArgs& a, hipStream_t stream) {
       default: return false;
     }
   }
-  switch (mt * 10 + conv_lds_waves()) {
-    case 14: launch_conv_lds<EL, CHUNKS, 1, 4>(a, stream); return true;
-    case 18: launch_conv_lds<EL, CHUNKS, 1, 8>(a, stream); return true;
-    case 24: launch_conv_lds<EL, CHUNKS, 2, 4>(a, stream); return true;
-    case 28: launch_conv_lds<EL, CHUNKS, 2, 8>(a, stream); return true;
-    case 44: launch_conv_lds<EL, CHUNKS, 4, 4>(a, stream); return true;
-    case 48: launch_conv_lds<EL, CHUNKS, 4, 8>(a, stream); return true;
+  switch (mt) {
+    case 1: launch_conv_lds<EL, CHUNKS, 1, 4>(a, stream); return true;
+    case 2: launch_conv_lds<EL, CHUNKS, 2, 8>(a, stream); return true;
+    case 4: launch_conv_lds<EL, CHUNKS, 4, 8>(a, stream); return true;
     default: return false;
   }
 }
@@ -2108,7 +2193,8 @@ int scn_hash_build(uint64_t* table_dev, size_t capacity, const int32_t* indices_
   Int3 g{{grid[0], grid[1], grid[2]}};
   if (n) {
     hipLaunchKernelGGL(k_hash_insert, dim3(ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, table_dev,
-                       (uint32_t)(capacity - 1), (const int4*)indices_dev, n, n_dev, g, (uint32_t*)nullptr);
+                       (uint32_t)(capacity - 1), (const int4*)indices_dev, n, n_dev, g, (uint32_t*)nullptr,
+                       (uint32_t*)nullptr);
     SCN_HIP(hipGetLastError());
   }
   return SCN_OK;

@@ -16,13 +16,17 @@ struct CoordLookup {
   const uint32_t* bitmap = nullptr;
   const uint32_t* prefix = nullptr;
   uint32_t rank_cap = 0;  // ranks >= rank_cap were truncated away
+  const uint32_t* filter = nullptr;  // hash lookups: occupancy bitmap tested before probing (nullable)
 };
 
 struct CoordTable {
   DevBuf buf;
   size_t cap = 0;     // allocated slots, power of two
   uint32_t mask = 0;  // slots in use - 1 (power of two <= cap), set by the last build
+  DevBuf filter;             // occupancy bitmap of the grid (optional, see alloc_filter)
+  size_t filter_words = 0;
   bool alloc_for(uint32_t max_rows);
+  bool alloc_filter(const int grid[3]);
   uint64_t* slots() const { return buf.as<uint64_t>(); }
   CoordLookup lookup() const;
 };
@@ -82,7 +86,7 @@ struct ConvWeights {
   uint32_t cin_pad = 0;  // padded input channels the kernel expects (elements)
   DevBuf wfrag;     // [steps][mtiles][64] x 16 bytes, MFMA A-operand order
   int mtiles32 = 0, steps32 = 0;
-  DevBuf zrow;      // 512 bytes of zeros
+  DevBuf zrow;      // 512 bytes of zeros, then 64 words of -1
   DevBuf wfrag32;   // cout > 16: [steps32][mtiles32][64] x 16 bytes, A-operand order of the 32x32 MFMA
   DevBuf wscale;    // fp32 [cout_pad]: s_w[c] (int8) or 1
   DevBuf bias;      // fp32 [cout_pad]
