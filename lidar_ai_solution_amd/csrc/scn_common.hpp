@@ -40,6 +40,40 @@ void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
   } while (0)
 
 // Owning device allocation.  alloc() returns false (and sets the error) on failure.
+// Pinned host memory that kernels can write (hipHostMalloc: mapped into the device address space).
+struct HostBuf {
+  void* p = nullptr;
+  HostBuf() = default;
+  HostBuf(const HostBuf&) = delete;
+  HostBuf& operator=(const HostBuf&) = delete;
+  HostBuf(HostBuf&& o) noexcept : p(o.p) { o.p = nullptr; }
+  HostBuf& operator=(HostBuf&& o) noexcept {
+    if (this != &o) {
+      release();
+      p = o.p;
+      o.p = nullptr;
+    }
+    return *this;
+  }
+  ~HostBuf() { release(); }
+  bool alloc(size_t n) {
+    release();
+    if (hipHostMalloc(&p, n ? n : 16, hipHostMallocDefault) != hipSuccess) {
+      p = nullptr;
+      return false;
+    }
+    return true;
+  }
+  void release() {
+    if (p) (void)hipHostFree(p);
+    p = nullptr;
+  }
+  template <class T>
+  T* as() const {
+    return static_cast<T*>(p);
+  }
+};
+
 struct DevBuf {
   void* p = nullptr;
   size_t bytes = 0;

@@ -867,7 +867,8 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
         io.b_requant_range = st.b_rq;
         io.relu_after_add = st.relu2;
       }
-      return conv_forward(*e.convs[st.conv], s.rb.nbr.as<int32_t>(), s.rb.ld, s.rb.n_out_dev(), s.rb.n_bound_out, io,
+      return conv_forward(*e.convs[st.conv], s.rb.nbr.as<int32_t>(), s.rb.ld, s.rb.n_out_dev(), s.rb.n_bound_out,
+                          s.rb.n_out_hint(), io,
                           stream);
     }
     case StepKind::Add: {

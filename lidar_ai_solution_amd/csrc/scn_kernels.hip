@@ -391,12 +391,16 @@ __device__ __forceinline__ int32_t coord_row(const CoordLookup& lk, uint32_t key
 // Thread (0,0) also publishes the row count for the kernels that follow (n_publish, nullable).
 __global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_coords, const uint32_t* n_out_dev,
                                                    uint32_t n_bound, GeomDev g, CoordLookup lk, int32_t* nbr,
-                                                   uint32_t ld, int identity_center, uint32_t* n_publish) {
+                                                   uint32_t ld, int identity_center, uint32_t* n_publish,
+                                                   uint32_t* n_host) {
   const uint32_t n = eff_n(n_out_dev, n_bound);
   const uint32_t o = blockIdx.x * 256 + threadIdx.x;
-  if (n_publish && o == 0 && blockIdx.y == 0) {
-    n_publish[0] = n;
-    n_publish[1] = n;
+  if (o == 0 && blockIdx.y == 0) {
+    if (n_publish) {
+      n_publish[0] = n;
+      n_publish[1] = n;
+    }
+    if (n_host) *n_host = n;  // pinned host word: the row count as a launch hint for the next forward
   }
   if (o >= n) return;
   const int k0 = blockIdx.y;
@@ -469,7 +473,17 @@ __global__ __launch_bounds__(256) void k_mark_outputs(const int4* __restrict__ i
   agg_flush(akeys, avals, bitmap);
 }
 
+// Row count of the previous build as seen by the host (0 before the first one has run): a hint for
+// launch configuration only, never used for bounds.
+uint32_t Rulebook::n_out_hint() const {
+  if (!host_count.p) return n_bound_out;
+  const uint32_t v = *reinterpret_cast<const volatile uint32_t*>(host_count.p);
+  return v == 0 || v > n_bound_out ? n_bound_out : v;
+}
+
 bool Rulebook::init(uint32_t max_in_, uint32_t max_out_, int kvol) {
+  if (!host_count.alloc(16)) return false;
+  memset(host_count.p, 0, 16);
   max_in = max_in_;
   max_out = max_out_;
   kvol_cap = kvol;
@@ -509,7 +523,7 @@ static int launch_build_nbr(const Rulebook& rb, const int32_t* out_coords, const
   const uint32_t blocks = n_bound ? ceil_div(n_bound, 256) : 1;  // one block even when empty: it publishes the count
   hipLaunchKernelGGL(k_build_nbr, dim3(blocks, rb.geom.ks[0]), dim3(256), 0, stream, (const int4*)out_coords, n_dev,
                      n_bound, to_dev(rb.geom), rb.in_lookup, rb.nbr.as<int32_t>(), rb.ld, identity_center ? 1 : 0,
-                     n_publish);
+                     n_publish, rb.host_count.as<uint32_t>());
   SCN_HIP(hipGetLastError());
   return SCN_OK;
 }
@@ -769,8 +783,7 @@ struct ConvArgs {
   float a_rq_s, a_rq_r;     // re-quantisation of an fp16 operand by an int8 Add (0 = none)
   float b_rq_s, b_rq_r;
   int relu2;
-  const char* zrow;  // >= 256 bytes of zeros (gather source of lanes without a neighbour)
-  int debug;  // measurement knob: 1 = no gathers, 2 = no weight slab loads, 8 = no epilogue, 16 = no main loop
+  const char* zrow;  // 512 bytes of zeros (gather source of lanes without a neighbour), then 64 words of -1
 };
 
 // int8 store of the fake-quant form: round(y * (127/amax)), saturated to +-127
@@ -976,175 +989,6 @@ __global__ __launch_bounds__(256) void k_conv_rows(const ConvArgs a) {
   }
 }
 
-constexpr int kConvMaxKvol = 27;  // largest kernel volume the workgroup kernel keeps in LDS
-
-// Workgroup kernel: 4 waves, each owning 16*NT output rows and all MT*16 output channels.
-//   * the weight slab of one iteration (one kernel offset when a row has >= 4 chunks, else 4/CHUNKS
-//     offsets) is staged through LDS once per workgroup, double-buffered, and read back as MFMA A
-//     fragments with ds_read_b128 (its own wait counter, so it never blocks on the gathers);
-//   * gathered rows go from global memory straight into the MFMA B operand, one iteration ahead;
-//   * neighbour indices are fetched two iterations ahead.
-// So during the MFMAs of iteration i the gathers and the weight slab of i+1 and the indices of i+2
-// are in flight.  Loaded values are only touched (masked, stored) in the iteration that consumes
-// them: any earlier ALU use would make the wave wait for the load right where it was issued.
-template <int EL, int CHUNKS, int MT, int NT>
-__global__ __launch_bounds__(256, 2) void k_conv_wg(const ConvArgs a) {
-  using Acc = typename Mma<EL>::Acc;
-  constexpr int SPK = CHUNKS >= 4 ? CHUNKS / 4 : 1;  // K-steps per iteration
-  constexpr int SLAB = SPK * MT * 64;                 // 16-byte fragments per iteration
-  constexpr int WPT = (SLAB + 255) / 256;             // fragments staged per thread
-  constexpr int R = 64 * NT;                          // output rows per workgroup
-  __shared__ v4i lds[2][SLAB];
-  __shared__ int32_t lidx[kConvMaxKvol * R];          // neighbour rows of the whole tile, all offsets
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int lr = lane & 15, lg = lane >> 4;
-  const uint32_t n = eff_n(a.n_out_dev, a.n_bound);
-  uint32_t tile;
-  if (!xcd_tile(n, 64u * NT, &tile)) return;  // uniform for the whole workgroup
-  const uint32_t row0 = (tile * 4 + wave) * (16 * NT);
-  // The neighbour table is read exactly once, so every one of its loads misses the caches.  Fetch the
-  // tile's whole block (kvol x R indices) up front with all loads in flight together, instead of
-  // paying that latency once per kernel offset inside the pipelined loop.
-  {
-    const uint32_t tile_row0 = tile * R;
-    const int total = a.kvol * R;
-    for (int base = 0; base < total; base += 256 * 8) {
-      int32_t tmp[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int f = base + j * 256 + tid;
-        const int k = f / R, r = f - k * R;
-        const bool v = f < total && tile_row0 + r < n;
-        tmp[j] = v ? a.nbr[(size_t)k * a.nbr_ld + tile_row0 + r] : -1;
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int f = base + j * 256 + tid;
-        if (f < total) lidx[f] = tmp[j];
-      }
-    }
-  }
-  __syncthreads();
-  const int32_t* __restrict__ my_idx = lidx + wave * (16 * NT) + lr;
-  const int iters = CHUNKS >= 4 ? a.kvol : a.steps;
-  const int total_chunks = a.kvol * CHUNKS;
-  const char* __restrict__ xb = a.x;
-  const v4i* __restrict__ wsrc = reinterpret_cast<const v4i*>(a.wfrag);
-  const uint32_t ldb = a.x_ld_bytes;
-  uint32_t rows[NT];
-  bool rvalid[NT];
-#pragma unroll
-  for (int u = 0; u < NT; ++u) {
-    rows[u] = row0 + u * 16 + lr;
-    rvalid[u] = rows[u] < n;
-  }
-
-  Acc acc[MT][NT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t)
-#pragma unroll
-    for (int u = 0; u < NT; ++u) acc[t][u] = Acc{0, 0, 0, 0};
-
-  int32_t idx0[NT], idx1[NT], idx2[NT];
-  v4i bcur[SPK][NT], bnext[SPK][NT];
-  v4i wreg[WPT];
-  const v4i vzero = {0, 0, 0, 0};
-
-// does this lane's slot of iteration IT exist at all (known without any load)
-#define SCN_SLOT_VALID(IT) ((IT) < iters && (CHUNKS >= 4 || 4 * (IT) + lg < total_chunks))
-#define SCN_SLOT_K(IT) (CHUNKS >= 4 ? (IT) : (4 * (IT) + lg) / CHUNKS)
-// neighbour indices of iteration IT from the LDS copy (rows beyond n hold -1 there)
-#define SCN_LOAD_IDX(IT, DST)                                                 \
-  {                                                                           \
-    const int k_ = SCN_SLOT_VALID(IT) ? SCN_SLOT_K(IT) : 0;                   \
-    _Pragma("unroll") for (int u = 0; u < NT; ++u) DST[u] = my_idx[k_ * R + u * 16]; \
-  }
-// unconditional gathers (row 0 for lanes without a neighbour); masked to zero when consumed
-#define SCN_GATHER(IT, IDX, DST)                                                            \
-  {                                                                                         \
-    const bool sv_ = SCN_SLOT_VALID(IT);                                                    \
-    _Pragma("unroll") for (int u = 0; u < NT; ++u) {                                        \
-      const bool ok_ = sv_ && rvalid[u] && IDX[u] >= 0;                                     \
-      const char* p_ = xb + (size_t)(ok_ ? (uint32_t)IDX[u] : 0u) * ldb;                    \
-      _Pragma("unroll") for (int ss = 0; ss < SPK; ++ss) {                                  \
-        const int c_ = CHUNKS >= 4 ? ss * 4 + lg : (4 * (IT) + lg) % CHUNKS;                \
-        DST[ss][u] = *reinterpret_cast<const v4i*>(p_ + c_ * 16);                           \
-      }                                                                                     \
-    }                                                                                       \
-  }
-#define SCN_LOAD_SLAB(IT)                                                     \
-  {                                                                           \
-    _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                         \
-      const int f_ = tid + j * 256;                                           \
-      if (SLAB % 256 == 0 || f_ < SLAB) wreg[j] = wsrc[(size_t)(IT) * SLAB + f_]; \
-    }                                                                         \
-  }
-#define SCN_STORE_SLAB(BUF)                                                   \
-  {                                                                           \
-    _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                         \
-      const int f_ = tid + j * 256;                                           \
-      if (SLAB % 256 == 0 || f_ < SLAB) lds[BUF][f_] = wreg[j];               \
-    }                                                                         \
-  }
-
-  SCN_LOAD_IDX(0, idx0);
-  SCN_LOAD_IDX(1, idx1);
-  SCN_LOAD_SLAB(0);
-  SCN_GATHER(0, idx0, bcur);
-  SCN_STORE_SLAB(0);
-  __syncthreads();
-  for (int it = 0; it < ((a.debug & 16) ? 0 : iters); ++it) {
-    SCN_LOAD_IDX(it + 2, idx2);
-    const bool more = it + 1 < iters;
-    if (more) {
-      if (!(a.debug & 2)) SCN_LOAD_SLAB(it + 1);
-      if (!(a.debug & 1)) SCN_GATHER(it + 1, idx1, bnext);
-    }
-    // MFMAs are unconditional: a branch around them makes the compiler shuttle all accumulators
-    // between AGPRs and VGPRs every iteration, which costs far more than multiplying by zero.
-    {
-      const bool sv = SCN_SLOT_VALID(it);
-      const v4i* la = lds[it & 1] + lane;
-#pragma unroll
-      for (int ss = 0; ss < SPK; ++ss) {
-        v4i bm[NT];
-#pragma unroll
-        for (int u = 0; u < NT; ++u) bm[u] = (sv && rvalid[u] && idx0[u] >= 0) ? bcur[ss][u] : vzero;
-#pragma unroll
-        for (int t = 0; t < MT; ++t) {
-          v4i av = vzero;
-          if (!(a.debug & 32)) av = la[(ss * MT + t) * 64];
-#pragma unroll
-          for (int u = 0; u < NT; ++u) acc[t][u] = Mma<EL>::run(av, bm[u], acc[t][u]);
-        }
-      }
-    }
-    if (more) SCN_STORE_SLAB((it + 1) & 1);
-    if (!(a.debug & 64)) __syncthreads();
-#pragma unroll
-    for (int u = 0; u < NT; ++u) {
-      idx0[u] = idx1[u];
-      idx1[u] = idx2[u];
-#pragma unroll
-      for (int ss = 0; ss < SPK; ++ss) bcur[ss][u] = bnext[ss][u];
-    }
-  }
-#undef SCN_SLOT_VALID
-#undef SCN_SLOT_K
-#undef SCN_LOAD_IDX
-#undef SCN_GATHER
-#undef SCN_LOAD_SLAB
-#undef SCN_STORE_SLAB
-  if (a.debug & 8) return;
-#pragma unroll
-  for (int u = 0; u < NT; ++u) {
-    if (!rvalid[u]) continue;
-#pragma unroll
-    for (int t = 0; t < MT; ++t) epilogue_store<EL>(a, rows[u], t * 16 + lg * 4, acc[t][u]);
-  }
-}
-
 // --------------------------------------------------------------------------------------------
 // 32x32 MFMA variant (output channels >= 32).
 // Measured issue rates on MI355X (independent accumulators, 4 waves per SIMD): v_mfma_i32_32x32x32_i8
@@ -1154,7 +998,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_wg(const ConvArgs a) {
 //                            B (K x 32): lane l supplies col n = l % 32, the 16 bytes of K-half l / 32
 //                            D (32 x 32): lane l holds col n = l % 32, rows 8 * (j / 4) + 4 * (l / 32) + j % 4
 // Rows of A are output channels, columns of B voxels; K-step s consumes chunks 2s and 2s+1 of the
-// (offset, chunk) sequence.  Otherwise the pipeline is that of k_conv_wg.
+// (offset, chunk) sequence.
 template <int EL>
 struct Mma32;
 template <>
@@ -1173,190 +1017,6 @@ struct Mma32<1> {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
   }
 };
-
-template <int EL, int CHUNKS, int MT, int NT>
-__global__ __launch_bounds__(256, 2) void k_conv32(const ConvArgs a) {
-  using Acc = typename Mma32<EL>::Acc;
-  using Acc4 = typename Mma32<EL>::Acc4;
-  constexpr int IPO = CHUNKS > 8 ? CHUNKS / 8 : 1;            // iterations per kernel offset
-  constexpr int SPK = CHUNKS >= 2 ? (CHUNKS / 2) / IPO : 1;   // K-steps per iteration
-  constexpr int SLAB = SPK * MT * 64;                         // 16-byte fragments per iteration
-  constexpr int WPT = (SLAB + 255) / 256;
-  constexpr int R = 128 * NT;                                 // output rows per workgroup
-  __shared__ v4i lds[3][SLAB];
-  __shared__ int32_t lidx[kConvMaxKvol * R];
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
-  const int ln = lane & 31, lh = lane >> 5;
-  const uint32_t n = eff_n(a.n_out_dev, a.n_bound);
-  uint32_t tile;
-  if (!xcd_tile(n, R, &tile)) return;
-  const uint32_t row0 = (tile * 4 + wave) * (32 * NT);
-  {
-    const uint32_t tile_row0 = tile * R;
-    const int total = a.kvol * R;
-    for (int base = 0; base < total; base += 256 * 8) {
-      int32_t tmp[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int f = base + j * 256 + tid;
-        const int k = f / R, r = f - k * R;
-        const bool v = f < total && tile_row0 + r < n;
-        tmp[j] = v ? a.nbr[(size_t)k * a.nbr_ld + tile_row0 + r] : -1;
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int f = base + j * 256 + tid;
-        if (f < total) lidx[f] = tmp[j];
-      }
-    }
-  }
-  __syncthreads();
-  const int32_t* __restrict__ my_idx = lidx + wave * (32 * NT) + ln;
-  const int iters = CHUNKS >= 2 ? a.kvol * IPO : (a.kvol + 1) / 2;
-  const char* __restrict__ xb = a.x;
-  const v4i* __restrict__ wsrc = reinterpret_cast<const v4i*>(a.wfrag);
-  const uint32_t ldb = a.x_ld_bytes;
-  uint32_t rows[NT];
-#pragma unroll
-  for (int u = 0; u < NT; ++u) rows[u] = row0 + u * 32 + ln;
-
-  Acc acc[MT][NT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t)
-#pragma unroll
-    for (int u = 0; u < NT; ++u)
-#pragma unroll
-      for (int j = 0; j < 16; ++j) acc[t][u][j] = 0;
-
-  // Software pipeline, steady state of iteration i:
-  //   issue   weight slab i+2 -> registers, gathers of i+1 -> registers, neighbour rows of i+2 <- LDS
-  //   compute MFMAs of i on the gathers issued during i-1 and the slab in LDS buffer i % 2
-  //   store   weight slab i+1 (loaded during i-1) -> LDS buffer (i+1) % 2, barrier
-  // Nothing in the loop is conditional and no loaded register is copied: the wave's memory counter
-  // retires loads in order, so a branch around a load (or a register move of a load's result)
-  // makes the compiler wait for *all* outstanding loads where the result is first touched, and the
-  // prefetch distance collapses to zero.  Hence the loop is unrolled by two with ping-pong register
-  // sets, and iterations past the end re-load the last slab / row 0 instead of skipping the loads.
-  int32_t idx0[NT], idx1[NT], idx2[NT];
-  v4i bA[SPK][NT], bB[SPK][NT];
-  v4i wA[WPT], wB[WPT];
-  const v4i vzero = {0, 0, 0, 0};
-  const int last = iters - 1;
-
-// does this lane's slot of iteration IT exist (known without any load), and its kernel offset
-#define SCN_SLOT_VALID(IT) ((IT) < iters && (CHUNKS >= 2 || 2 * (IT) + lh < a.kvol))
-#define SCN_SLOT_K(IT) (CHUNKS >= 2 ? (IT) / IPO : 2 * (IT) + lh)
-// neighbour rows of iteration IT from the LDS copy (rows beyond n hold -1 there)
-#define SCN_LOAD_IDX(IT, DST)                                                              \
-  {                                                                                        \
-    const int k_ = SCN_SLOT_VALID(IT) ? SCN_SLOT_K(IT) : 0;                                \
-    _Pragma("unroll") for (int u = 0; u < NT; ++u) DST[u] = my_idx[k_ * R + u * 32];       \
-  }
-// unconditional gathers (row 0 for lanes without a neighbour); masked to zero when consumed
-#define SCN_GATHER(IT, IDX, DST)                                                           \
-  {                                                                                        \
-    const bool sv_ = SCN_SLOT_VALID(IT);                                                   \
-    const int sub_ = CHUNKS >= 2 ? ((IT) % IPO) * (2 * SPK) : 0;                           \
-    _Pragma("unroll") for (int u = 0; u < NT; ++u) {                                       \
-      const bool ok_ = sv_ && IDX[u] >= 0;                                                 \
-      const char* p_ = xb + (size_t)(ok_ ? (uint32_t)IDX[u] : 0u) * ldb;                   \
-      _Pragma("unroll") for (int ss = 0; ss < SPK; ++ss) {                                 \
-        const int c_ = CHUNKS >= 2 ? sub_ + 2 * ss + lh : 0;                               \
-        DST[ss][u] = *reinterpret_cast<const v4i*>(p_ + c_ * 16);                          \
-      }                                                                                    \
-    }                                                                                      \
-  }
-#define SCN_LOAD_SLAB(IT, W)                                                               \
-  {                                                                                        \
-    const int it_ = (IT) < last ? (IT) : last;                                             \
-    _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                                      \
-      const int f_ = tid + j * 256;                                                        \
-      W[j] = wsrc[(size_t)it_ * SLAB + ((SLAB % 256 == 0 || f_ < SLAB) ? f_ : 0)];         \
-    }                                                                                      \
-  }
-#define SCN_STORE_SLAB(BUF, W)                                                             \
-  {                                                                                        \
-    _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                                      \
-      const int f_ = tid + j * 256;                                                        \
-      if (SLAB % 256 == 0 || f_ < SLAB) lds[BUF][f_] = W[j];                               \
-    }                                                                                      \
-  }
-// one iteration: CUR / NXT / NN = LDS buffers of slabs IT, IT+1, IT+2 (indices mod 3)
-#define SCN_ITER(IT, BC, BN, WC, WN)                                                       \
-  {                                                                                        \
-    SCN_LOAD_IDX((IT) + 2, idx2);                                                          \
-    SCN_LOAD_SLAB((IT) + 3, WN);                                                           \
-    SCN_GATHER((IT) + 1, idx1, BN);                                                        \
-    __builtin_amdgcn_sched_barrier(0);                                                     \
-    const bool sv = SCN_SLOT_VALID(IT);                                                    \
-    const int nxt_ = cur == 2 ? 0 : cur + 1;                                               \
-    const int nn_ = nxt_ == 2 ? 0 : nxt_ + 1;                                              \
-    const v4i* la = &lds[nxt_][0] + lane;                                                  \
-    _Pragma("unroll") for (int ss = 0; ss < SPK; ++ss) {                                   \
-      v4i bm[NT];                                                                          \
-      _Pragma("unroll") for (int u = 0; u < NT; ++u)                                       \
-        bm[u] = (sv && idx0[u] >= 0) ? BC[ss][u] : vzero;                                  \
-      _Pragma("unroll") for (int t = 0; t < MT; ++t)                                       \
-        _Pragma("unroll") for (int u = 0; u < NT; ++u)                                     \
-          acc[t][u] = Mma32<EL>::run(af[ss][t], bm[u], acc[t][u]);                         \
-      /* the same K-step of the next iteration, from the slab stored one iteration ago */  \
-      _Pragma("unroll") for (int t = 0; t < MT; ++t) af[ss][t] = la[(ss * MT + t) * 64];   \
-      __builtin_amdgcn_sched_barrier(0); /* keep the refill here: the scheduler sinks it to its use */ \
-    }                                                                                      \
-    SCN_STORE_SLAB(nn_, WC);                                                               \
-    __syncthreads();                                                                       \
-    cur = nxt_;                                                                            \
-    _Pragma("unroll") for (int u = 0; u < NT; ++u) {                                       \
-      idx0[u] = idx1[u];                                                                   \
-      idx1[u] = idx2[u];                                                                   \
-    }                                                                                      \
-  }
-
-  v4i af[SPK][MT];  // A fragments of the current iteration, refilled one iteration ahead
-  int cur = 0;
-  SCN_LOAD_IDX(0, idx0);
-  SCN_LOAD_IDX(1, idx1);
-  SCN_LOAD_SLAB(0, wA);
-  SCN_LOAD_SLAB(1, wB);
-  SCN_GATHER(0, idx0, bA);
-  SCN_STORE_SLAB(0, wA);
-  SCN_STORE_SLAB(1, wB);
-  SCN_LOAD_SLAB(2, wB);
-  __syncthreads();
-#pragma unroll
-  for (int ss = 0; ss < SPK; ++ss)
-#pragma unroll
-    for (int t = 0; t < MT; ++t) af[ss][t] = lds[0][(ss * MT + t) * 64 + lane];
-  int it = 0;
-  for (; it + 1 < iters; it += 2) {
-    SCN_ITER(it, bA, bB, wB, wA);
-    SCN_ITER(it + 1, bB, bA, wA, wB);
-  }
-  if (it < iters) SCN_ITER(it, bA, bB, wB, wA);
-#undef SCN_SLOT_VALID
-#undef SCN_SLOT_K
-#undef SCN_LOAD_IDX
-#undef SCN_GATHER
-#undef SCN_LOAD_SLAB
-#undef SCN_STORE_SLAB
-#undef SCN_ITER
-  if (a.debug & 8) return;
-  const int cout_pad = (a.cout + 15) & ~15;
-#pragma unroll
-  for (int u = 0; u < NT; ++u) {
-    if (rows[u] >= n) continue;
-#pragma unroll
-    for (int t = 0; t < MT; ++t)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int co = t * 32 + g * 8 + lh * 4;
-        if (co >= cout_pad) continue;
-        const Acc4 piece = {acc[t][u][4 * g], acc[t][u][4 * g + 1], acc[t][u][4 * g + 2], acc[t][u][4 * g + 3]};
-        epilogue_store<EL>(a, rows[u], co, piece);
-      }
-  }
-}
 
 // --------------------------------------------------------------------------------------------
 // LDS-staged gather kernel (32x32 MFMA, output channels >= 32).
@@ -1378,8 +1038,11 @@ __global__ __launch_bounds__(256, 2) void k_conv32(const ConvArgs a) {
 //                   so those need a wait on the wave's own memory counter only
 // The memory counter retires loads in order, so "at most N outstanding" names exactly which older load
 // has landed.  Issue order per iteration i: slab S(i+1), indices I(i+4), gathers G(i+1).
+// waves per SIMD the kernel is compiled for: two 8-wave workgroups per CU, or one of 10 / 12 waves
+constexpr int conv_lds_min_waves(int waves) { return waves <= 8 ? 4 : 3; }
+
 template <int EL, int CHUNKS, int MT, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, 4) void k_conv_lds(const ConvArgs a) {
+__global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_lds(const ConvArgs a) {
   using Acc = typename Mma32<EL>::Acc;
   using Acc4 = typename Mma32<EL>::Acc4;
   constexpr int THREADS = 64 * WAVES;
@@ -1388,13 +1051,15 @@ __global__ __launch_bounds__(64 * WAVES, 4) void k_conv_lds(const ConvArgs a) {
   constexpr int G = 8 / SEG;                     // kernel offsets per iteration
   constexpr int RP = 8 / SEG;                    // rows per 128 bytes of the gathered stage
   constexpr int SLAB = 4 * MT * 64;              // 16-byte weight fragments per iteration
-  static_assert(SLAB % THREADS == 0, "every wave must issue the same number of slab loads");
-  constexpr int WPT = SLAB / THREADS;            // slab loads per wave and iteration
+  constexpr int NL = SLAB / 64;                  // 1 KB wave-loads per slab
+  constexpr int WPT = (NL + WAVES - 1) / WAVES;  // slab loads per wave and iteration (the same for every wave:
+                                                 // the waits below count loads; surplus ones go to `spare`)
   constexpr int IDXI = G >= 2 ? G / 2 : 1;       // index loads per wave and iteration (64 entries each)
   constexpr int R = 32 * WAVES;                  // output rows per workgroup
   __shared__ v4i lds[2][SLAB];
   __shared__ v4i ring[WAVES][256];
   __shared__ int32_t iring[4][WAVES][64 * IDXI];
+  __shared__ v4i spare[NL % WAVES ? 64 : 1];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int ln = lane & 31, lh = lane >> 5;
@@ -1425,9 +1090,15 @@ __global__ __launch_bounds__(64 * WAVES, 4) void k_conv_lds(const ConvArgs a) {
 #define SCN_SLAB(IT)                                                                            \
   {                                                                                             \
     const int it_ = (IT) < iters ? (IT) : iters - 1;                                            \
-    _Pragma("unroll") for (int j = 0; j < WPT; ++j)                                             \
-      __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + (size_t)it_ * SLAB + j * THREADS + tid), \
-                                       (lptr_t)&lds[(IT) & 1][j * THREADS + wave * 64], 16, 0, 0); \
+    _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                                           \
+      const int f_ = j * WAVES + wave; /* wave-uniform */                                       \
+      if (NL % WAVES == 0 || f_ < NL)                                                           \
+        __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + (size_t)it_ * SLAB + f_ * 64 + lane),  \
+                                         (lptr_t)&lds[(IT) & 1][f_ * 64], 16, 0, 0);            \
+      else                                                                                      \
+        __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + (size_t)it_ * SLAB + lane),            \
+                                         (lptr_t)&spare[0], 16, 0, 0);                          \
+    }                                                                                           \
   }
 // neighbour rows of iteration IT -> index ring stage IT % 4: entry e = 64 q + lane is kernel offset
 // e / 32 of the iteration, tile row e % 32; slots outside the volume or beyond row n read -1
@@ -1539,7 +1210,7 @@ __global__ __launch_bounds__(64 * WAVES, 4) void k_conv_lds(const ConvArgs a) {
     SCN_READ_INDEX((it + 1) & 3, gi);
     SCN_GATHER(it + 1, gi);
     const uint32_t la = lds_a_addr + (uint32_t)(it & 1) * (SLAB * 16);
-    if constexpr (MT >= 4) {
+    if constexpr (MT >= 4 && conv_lds_min_waves(WAVES) >= 4) {
       // 64 accumulator registers leave room for one set of fragments under the 128-register budget of
       // four waves per SIMD (a spill would also put scratch loads into the memory counter and break the
       // counts above); the other three waves of the SIMD cover the LDS latency instead
@@ -1653,7 +1324,7 @@ bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* 
       }
   // 32x32 MFMA order for layers with more than 16 output channels: [step][mtile32][lane] x 16 bytes,
   // lane l = channel 32 t + l % 32, K-half l / 32; K-step s holds chunks 2s, 2s+1 of the sequence
-  if (mtiles >= 2) {
+  if (mtiles >= 1) {
     mtiles32 = (cout + 31) / 32;
     if (mtiles32 == 3) mtiles32 = 4;  // kernels exist for 1, 2 and 4 tiles; the fourth is zero weights
     steps32 = 4 * ((kvol * chunks + 7) / 8);  // whole iterations of 4 K-steps, zero weights beyond the volume
@@ -1698,48 +1369,22 @@ bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* 
   return true;
 }
 
-// 0: workgroup kernel (LDS-staged weights, software-pipelined gathers); 1: plain row-split kernel.
-// The second is kept for A/B measurements (environment variable SCN_CONV_IMPL=rows).
+// SCN_CONV_IMPL=rows forces the plain row-split kernel (A/B measurements; it is also the fallback for
+// more than 128 output channels).
 static int conv_impl() {
   static const int impl = [] {
     const char* e = getenv("SCN_CONV_IMPL");
-    return (e && !strcmp(e, "rows")) ? 1 : (e && !strcmp(e, "wg16")) ? 2 : (e && !strcmp(e, "reg32")) ? 3 : 0;
+    return (e && !strcmp(e, "rows")) ? 1 : 0;
   }();
   return impl;
 }
 
 template <int EL, int CHUNKS, int MT>
 static void launch_conv_rows(const ConvArgs& a, hipStream_t stream) {
-  // Row tiles per wave: 4 up to 64 output channels, 2 for 128.  Measured on a 65.7 k-row 128->128
-  // layer: NT=2 58.6 us, NT=4 71.6 us (compiled for two workgroups per CU) -- with 4 the layer is only
-  // 257 workgroups, one wave per SIMD, and nothing hides the LDS and gather latency.
   constexpr int NT = MT >= 8 ? 2 : 4;
   const uint32_t rows_per_block = 4 * 16 * NT;
-  constexpr int SPK = CHUNKS >= 4 ? CHUNKS / 4 : 1;
-  constexpr bool lds_ok = 2 * SPK * MT * 64 * 16 + kConvMaxKvol * 64 * NT * 4 <= 64 * 1024;
   const uint32_t blocks = 8 * ceil_div(ceil_div(a.n_bound, rows_per_block), 8);  // see xcd_tile()
-  if (conv_impl() != 1 && lds_ok && a.kvol <= kConvMaxKvol) {
-    if constexpr (lds_ok)
-      hipLaunchKernelGGL((k_conv_wg<EL, CHUNKS, MT, NT>), dim3(blocks), dim3(256), 0, stream, a);
-  } else {
-    hipLaunchKernelGGL((k_conv_rows<EL, CHUNKS, MT, NT>), dim3(blocks), dim3(256), 0, stream, a);
-  }
-}
-
-// rows per wave of the 32x32 kernel, in 32-row tiles (environment variable SCN_CONV_NT, default 1)
-static int conv32_nt() {
-  static const int nt = [] {
-    const char* e = getenv("SCN_CONV_NT");
-    return (e && atoi(e) == 2) ? 2 : 1;
-  }();
-  return nt;
-}
-
-template <int EL, int CHUNKS, int MT, int NT>
-static void launch_conv32(const ConvArgs& a, hipStream_t stream) {
-  constexpr uint32_t R = 128 * NT;
-  const uint32_t blocks = 8 * ceil_div(ceil_div(a.n_bound, R), 8);  // see xcd_tile()
-  hipLaunchKernelGGL((k_conv32<EL, CHUNKS, MT, NT>), dim3(blocks), dim3(256), 0, stream, a);
+  hipLaunchKernelGGL((k_conv_rows<EL, CHUNKS, MT, NT>), dim3(blocks), dim3(256), 0, stream, a);
 }
 
 template <int EL, int CHUNKS, int MT, int WAVES>
@@ -1749,34 +1394,47 @@ static void launch_conv_lds(const ConvArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL((k_conv_lds<EL, CHUNKS, MT, WAVES>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
 }
 
-// SCN_CONV_IMPL=reg32 selects the register-gather 32x32 kernel
+// Workgroup size of the 128-channel kernel.  A layer of a lidar backbone's deep stages is about one
+// workgroup per CU, so its duration is that of the busiest CU: 257 tiles of 256 rows on 256 CUs take
+// as long as 512.  With the expected row count (the count of the previous forward, see
+// Rulebook::n_out_hint) the tile height is chosen so that all rows fit one workgroup per CU when they
+// can: 8, 10 or 12 waves of 32 rows; beyond 384 rows per CU it is 8 waves and two workgroups per CU.
+static int conv_lds_waves(uint32_t n_hint) {
+  static const int forced = [] {
+    const char* e = getenv("SCN_CONV_WAVES");
+    return e ? atoi(e) : 0;
+  }();
+  if (forced == 8 || forced == 10 || forced == 12) return forced;
+  constexpr uint32_t kCus = 256;
+  if (n_hint <= kCus * 256u) return 8;
+  if (n_hint <= kCus * 320u) return 10;
+  if (n_hint <= kCus * 384u) return 12;
+  return 8;
+}
+
 template <int EL, int CHUNKS>
-static bool dispatch_mt32(int mt, const ConvArgs& a, hipStream_t stream) {
-  if (conv_impl() == 3) {
-    const int nt = conv32_nt();
-    switch (mt * 10 + nt) {
-      case 11: launch_conv32<EL, CHUNKS, 1, 1>(a, stream); return true;
-      case 21: launch_conv32<EL, CHUNKS, 2, 1>(a, stream); return true;
-      case 41: launch_conv32<EL, CHUNKS, 4, 1>(a, stream); return true;
-      default: return false;
-    }
-  }
+static bool dispatch_mt32(int mt, uint32_t n_hint, const ConvArgs& a, hipStream_t stream) {
   switch (mt) {
     case 1: launch_conv_lds<EL, CHUNKS, 1, 4>(a, stream); return true;
     case 2: launch_conv_lds<EL, CHUNKS, 2, 8>(a, stream); return true;
-    case 4: launch_conv_lds<EL, CHUNKS, 4, 8>(a, stream); return true;
+    case 4:
+      switch (conv_lds_waves(n_hint)) {
+        case 10: launch_conv_lds<EL, CHUNKS, 4, 10>(a, stream); return true;
+        case 12: launch_conv_lds<EL, CHUNKS, 4, 12>(a, stream); return true;
+        default: launch_conv_lds<EL, CHUNKS, 4, 8>(a, stream); return true;
+      }
     default: return false;
   }
 }
 
 template <int EL>
-static bool dispatch_chunks32(int chunks, int mt, const ConvArgs& a, hipStream_t stream) {
+static bool dispatch_chunks32(int chunks, int mt, uint32_t n_hint, const ConvArgs& a, hipStream_t stream) {
   switch (chunks) {
-    case 1: return dispatch_mt32<EL, 1>(mt, a, stream);
-    case 2: return dispatch_mt32<EL, 2>(mt, a, stream);
-    case 4: return dispatch_mt32<EL, 4>(mt, a, stream);
-    case 8: return dispatch_mt32<EL, 8>(mt, a, stream);
-    case 16: return dispatch_mt32<EL, 16>(mt, a, stream);
+    case 1: return dispatch_mt32<EL, 1>(mt, n_hint, a, stream);
+    case 2: return dispatch_mt32<EL, 2>(mt, n_hint, a, stream);
+    case 4: return dispatch_mt32<EL, 4>(mt, n_hint, a, stream);
+    case 8: return dispatch_mt32<EL, 8>(mt, n_hint, a, stream);
+    case 16: return dispatch_mt32<EL, 16>(mt, n_hint, a, stream);
     default: return false;
   }
 }
@@ -1805,7 +1463,7 @@ static bool dispatch_chunks(int chunks, int mt, const ConvArgs& a, hipStream_t s
 }
 
 int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, const uint32_t* n_out_dev,
-                 uint32_t n_bound, const scn_conv_io& io, hipStream_t stream) {
+                 uint32_t n_bound, uint32_t n_hint, const scn_conv_io& io, hipStream_t stream) {
   if (n_bound == 0) return SCN_OK;
   const int esz = w.precision == SCN_PRECISION_INT8 ? 1 : 2;
   SCN_REQUIRE(io.x_dev && io.out_dev, SCN_ERR_INVALID, "conv: null input or output");
@@ -1865,16 +1523,13 @@ int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, cons
     SCN_REQUIRE(io.out_dynamic_range > 0.f, SCN_ERR_INVALID, "conv: int8 output needs out_dynamic_range > 0");
   if (w.precision == SCN_PRECISION_INT8)
     SCN_REQUIRE(io.x_dynamic_range > 0.f, SCN_ERR_INVALID, "conv: int8 input needs x_dynamic_range > 0");
-  {
-    const char* dbg = getenv("SCN_CONV_DEBUG");
-    a.debug = dbg ? atoi(dbg) : 0;
-  }
   bool ok = false;
   const int mt32 = w.mtiles32;
-  if (mt32 >= 1 && mt32 <= 4 && w.kvol <= kConvMaxKvol && (conv_impl() == 0 || conv_impl() == 3)) {
+  if (mt32 >= 1 && mt32 <= 4 && conv_impl() == 0) {
     a.wfrag = w.wfrag32.as<uint4>();
-    ok = w.precision == SCN_PRECISION_INT8 ? dispatch_chunks32<0>(w.chunks, mt32, a, stream)
-                                           : dispatch_chunks32<1>(w.chunks, mt32, a, stream);
+    if (n_hint == 0 || n_hint > n_bound) n_hint = n_bound;
+    ok = w.precision == SCN_PRECISION_INT8 ? dispatch_chunks32<0>(w.chunks, mt32, n_hint, a, stream)
+                                           : dispatch_chunks32<1>(w.chunks, mt32, n_hint, a, stream);
   }
   if (!ok) {
     a.wfrag = w.wfrag.as<uint4>();
@@ -2403,7 +2058,8 @@ int scn_conv_forward(const scn_conv* c, const scn_rulebook* rb, const scn_conv_i
   SCN_REQUIRE(rb->rb.built, SCN_ERR_INVALID, "scn_conv_forward: rulebook not built");
   SCN_REQUIRE(rb->rb.geom.kvol == c->w.kvol, SCN_ERR_INVALID, "scn_conv_forward: kernel volume mismatch (%d vs %d)",
               rb->rb.geom.kvol, c->w.kvol);
-  return conv_forward(c->w, rb->rb.nbr.as<int32_t>(), rb->rb.ld, rb->rb.n_out_dev(), rb->rb.n_bound_out, *io,
+  return conv_forward(c->w, rb->rb.nbr.as<int32_t>(), rb->rb.ld, rb->rb.n_out_dev(), rb->rb.n_bound_out,
+                      rb->rb.n_out_hint(), *io,
                       (hipStream_t)stream);
 }
 

@@ -55,6 +55,7 @@ struct Rulebook {
   uint32_t ld = 0;
   DevBuf out_idx;             // int32 [max_out][4] (strided)
   DevBuf counters;            // uint32: [0] n_out kept, [1] n_out before truncation, [2..] scratch
+  HostBuf host_count;         // pinned: [0] n_out kept of the last build that has run (launch hint)
   DevBuf bitmap, blocksum, prefix;  // strided: occupancy bitmap of the output grid, per-block popcounts, per-word ranks
   size_t bitmap_words = 0, bitmap_cap_words = 0;
   DevBuf pair_scratch;        // pair compaction: per (k, block) counts
@@ -74,6 +75,7 @@ struct Rulebook {
   CoordLookup out_lookup() const;  // strided: rows of the output tensor from bitmap ranks
   int pairs(int32_t* pair_in, int32_t* pair_out, int64_t* offsets, uint64_t capacity, hipStream_t stream);
   const uint32_t* n_out_dev() const { return counters.as<uint32_t>(); }
+  uint32_t n_out_hint() const;
 };
 
 // Packed weights of one convolution (= scn_conv of the C ABI).
@@ -93,8 +95,9 @@ struct ConvWeights {
   bool init(const uint16_t* w_fp16, const int shape[5], const float* ranges, const uint16_t* bias_fp16, int prec);
 };
 
+// n_hint: expected row count (0 = unknown), only used to choose the launch configuration
 int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, const uint32_t* n_out_dev,
-                 uint32_t n_bound, const scn_conv_io& io, hipStream_t stream);
+                 uint32_t n_bound, uint32_t n_hint, const scn_conv_io& io, hipStream_t stream);
 
 int set_count(uint32_t* dst, const uint32_t* n_dev, uint32_t n_bound, hipStream_t stream);
 int fill_u32(void* p, uint32_t value, size_t count, hipStream_t stream);
