@@ -783,6 +783,7 @@ struct ConvArgs {
   float a_rq_s, a_rq_r;     // re-quantisation of an fp16 operand by an int8 Add (0 = none)
   float b_rq_s, b_rq_r;
   int relu2;
+  int out_vec16;     // output rows are 16-byte aligned and a multiple of 16 bytes: 16-byte stores allowed
   const char* zrow;  // 512 bytes of zeros (gather source of lanes without a neighbour), then 64 words of -1
 };
 
@@ -830,10 +831,12 @@ __device__ __forceinline__ bool xcd_tile(uint32_t n, uint32_t rows_per_block, ui
   return j < per && *tile < tiles;
 }
 
-// Stores 4 consecutive channels of one row after the fused epilogue.
+// Fused epilogue of 4 consecutive channels of one row: bias, requantisation scale, ReLU, residual add
+// (with the mid-quantisation the un-fused graph would have applied), second ReLU.  Also dumps the raw
+// accumulators when asked to.  y[] receives the values to store.
 template <int EL>
-__device__ __forceinline__ void epilogue_store(const ConvArgs& a, uint32_t row, int co, const typename Mma<EL>::Acc& acc) {
-  float y[4];
+__device__ __forceinline__ void epilogue_values(const ConvArgs& a, uint32_t row, int co,
+                                                const typename Mma<EL>::Acc& acc, float y[4]) {
   const float4 bs = *reinterpret_cast<const float4*>(a.bias + co);
   const float b4[4] = {bs.x, bs.y, bs.z, bs.w};
   if (EL == 0) {
@@ -890,18 +893,32 @@ __device__ __forceinline__ void epilogue_store(const ConvArgs& a, uint32_t row, 
       y[j] = v;
     }
   }
-  if (a.out_dtype == SCN_DTYPE_INT8) {
-    char4 q;
-    q.x = (signed char)quant_f(y[0], a.out_r);
-    q.y = (signed char)quant_f(y[1], a.out_r);
-    q.z = (signed char)quant_f(y[2], a.out_r);
-    q.w = (signed char)quant_f(y[3], a.out_r);
-    *reinterpret_cast<char4*>(a.out + (size_t)row * a.out_ld + co) = q;
-  } else {
-    typedef _Float16 v4h __attribute__((ext_vector_type(4)));
-    v4h h = {(_Float16)y[0], (_Float16)y[1], (_Float16)y[2], (_Float16)y[3]};
-    *reinterpret_cast<v4h*>(reinterpret_cast<_Float16*>(a.out) + (size_t)row * a.out_ld + co) = h;
-  }
+}
+
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ char4 pack_int8(const ConvArgs& a, const float y[4]) {
+  char4 q;
+  q.x = (signed char)quant_f(y[0], a.out_r);
+  q.y = (signed char)quant_f(y[1], a.out_r);
+  q.z = (signed char)quant_f(y[2], a.out_r);
+  q.w = (signed char)quant_f(y[3], a.out_r);
+  return q;
+}
+
+__device__ __forceinline__ v4h pack_fp16(const float y[4]) {
+  return v4h{(_Float16)y[0], (_Float16)y[1], (_Float16)y[2], (_Float16)y[3]};
+}
+
+// Stores 4 consecutive channels of one row after the fused epilogue.
+template <int EL>
+__device__ __forceinline__ void epilogue_store(const ConvArgs& a, uint32_t row, int co, const typename Mma<EL>::Acc& acc) {
+  float y[4];
+  epilogue_values<EL>(a, row, co, acc, y);
+  if (a.out_dtype == SCN_DTYPE_INT8)
+    *reinterpret_cast<char4*>(a.out + (size_t)row * a.out_ld + co) = pack_int8(a, y);
+  else
+    *reinterpret_cast<v4h*>(reinterpret_cast<_Float16*>(a.out) + (size_t)row * a.out_ld + co) = pack_fp16(y);
 }
 
 // Row-split kernel: each wave owns 16*NT output rows and all MT*16 output channels; both operands
@@ -1253,18 +1270,66 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
 #undef SCN_SLAB
 #undef SCN_INDEX
 #undef SCN_GATHER
+  // Epilogue.  Each lane holds 4-channel pieces of one row; writing them directly would touch every
+  // 128-byte line of the tile 16 times.  The pieces go through the wave's LDS stage instead (same XOR
+  // placement as the gathers) and leave as 16 bytes per lane, 8 lanes per row.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stage still receives the gathers issued past the end
   const uint32_t row = row0 + ln;
-  if (row >= n) return;
   const int cout_pad = (a.cout + 15) & ~15;
+  if (!a.out_vec16) {
+    if (row >= n) return;
 #pragma unroll
-  for (int t = 0; t < MT; ++t)
+    for (int t = 0; t < MT; ++t)
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int co = t * 32 + g * 8 + lh * 4;
-      if (co >= cout_pad) continue;
-      const Acc4 piece = {acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
-      epilogue_store<EL>(a, row, co, piece);
+      for (int g = 0; g < 4; ++g) {
+        const int co = t * 32 + g * 8 + lh * 4;
+        if (co >= cout_pad) continue;
+        const Acc4 piece = {acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
+        epilogue_store<EL>(a, row, co, piece);
+      }
+    return;
+  }
+  char* stage = reinterpret_cast<char*>(&ring[wave][0]);
+  const bool out8 = a.out_dtype == SCN_DTYPE_INT8;
+  constexpr int PASSES = MT >= 4 ? 2 : 1;          // fp16 rows of 128 channels take two 128-byte passes
+  constexpr int TPP = MT >= 4 ? 2 : MT;            // 32-channel tiles per fp16 pass
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    if (out8 && p > 0) break;
+    const int t_lo = out8 ? 0 : p * TPP, t_hi = out8 ? MT : p * TPP + TPP;
+    const int c0 = t_lo * 32;                      // first channel of the pass
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      if (t < t_lo || t >= t_hi) continue;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int co = t * 32 + g * 8 + lh * 4;
+        if (co >= cout_pad || row >= n) continue;
+        const Acc4 piece = {acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
+        float y[4];
+        epilogue_values<EL>(a, row, co, piece, y);
+        const int off = (co - c0) * (out8 ? 1 : 2);  // byte offset inside the 128-byte pass row
+        char* dst = stage + ln * 128 + (((off >> 4) ^ (ln & 7)) << 4) + (off & 15);
+        if (out8)
+          *reinterpret_cast<char4*>(dst) = pack_int8(a, y);
+        else
+          *reinterpret_cast<v4h*>(dst) = pack_fp16(y);
+      }
     }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    const int osz = out8 ? 1 : 2;
+    const int valid = (cout_pad - c0) * osz;       // bytes of the pass row that exist
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int r = (lane >> 3) + 8 * j, c = lane & 7;
+      const uint32_t grow = row0 + r;
+      if (grow < n && c * 16 < valid) {
+        const v4i v = *reinterpret_cast<const v4i*>(stage + r * 128 + ((c ^ (r & 7)) << 4));
+        *reinterpret_cast<v4i*>(a.out + ((size_t)grow * a.out_ld + c0) * osz + c * 16) = v;
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
 }
 
 bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* ranges, const uint16_t* bias_fp16,
@@ -1519,6 +1584,8 @@ int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, cons
   a.b_rq_s = s_of(io.b_requant_range);
   a.b_rq_r = r_of(io.b_requant_range);
   a.relu2 = io.relu_after_add;
+  a.out_vec16 = (((size_t)io.out_ld * osz) % 16 == 0 && ((uintptr_t)io.out_dev & 15) == 0 &&
+                 ((size_t)((w.cout + 15) & ~15) * osz) % 16 == 0) ? 1 : 0;
   if (io.out_dtype == SCN_DTYPE_INT8)
     SCN_REQUIRE(io.out_dynamic_range > 0.f, SCN_ERR_INVALID, "conv: int8 output needs out_dynamic_range > 0");
   if (w.precision == SCN_PRECISION_INT8)
