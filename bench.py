@@ -99,7 +99,10 @@ def copy_probe():
 # HBM bytes per launch of the dominant kernel from hardware counters (rocprofv3 --pmc FETCH_SIZE, then
 # WRITE_SIZE, each scaled by what the same counter reads for the copy probe).  Keyed by everything the
 # figure depends on, so that any other workload reports null instead of a stale number.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    # int8 SubM 128->128 3x3x3 on the 65,699 rows of the default frame: FETCH_SIZE x 1.9999 + WRITE_SIZE x 1.0000
+    ("int8", (128, 128, 1, (3, 3, 3)), 123646): 41259536,
+}
 
 
 def stage_pair_counts(eng_keep, graph):
@@ -294,7 +297,7 @@ def main():
     # which roof bounds the kernel: its algorithmic intensity against the machine balance (ops per HBM byte)
     intensity = dom_ops / dom_bytes
     ridge = mfma_peak * 1e12 / (HBM_PEAK_GBS * 1e9)
-    kernel = (f"k_conv_wg {args.precision} Cin={dom_key[0]} Cout={dom_key[1]} {'subm' if dom_key[2] else 'strided'} "
+    kernel = (f"k_conv_lds {args.precision} Cin={dom_key[0]} Cout={dom_key[1]} {'subm' if dom_key[2] else 'strided'} "
               f"k={'x'.join(map(str, dom_key[3]))}")
     traffic = MEASURED_TRAFFIC.get((args.precision, dom_key, int(nvox)))
     common = {
