@@ -177,6 +177,7 @@ struct scn_engine {
   std::vector<std::unique_ptr<RbSlot>> rulebooks;
   std::vector<std::unique_ptr<ConvWeights>> convs;
   std::vector<Step> steps;
+  std::vector<char> dense_precleared;  // per step: its dense output was zeroed by the forward's batched fill
   std::map<std::string, int> tensor_by_name;
   // input binding
   const void* in_feat = nullptr;
@@ -797,7 +798,38 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
       c0.idx = e.in_idx;
       c0.n_bound = n;
       c0.has_lookup = false;
-      int rc = set_count(e.in_count.as<uint32_t>(), e.dds, n, stream);
+      // One launch publishes the clamped input count and clears everything this forward builds into:
+      // the input hash (+ its occupancy filter), the output bitmaps of the strided rulebooks and the
+      // dense outputs.  The steps that own those buffers then skip their own fills.
+      FillJob jobs[kMaxFillJobs];
+      int nj = 0;
+      auto add = [&](void* p, size_t words, uint32_t value) {
+        if (!p || words == 0 || nj >= kMaxFillJobs) return false;
+        jobs[nj++] = FillJob{p, words, value};
+        return true;
+      };
+      e.dense_precleared.assign(e.steps.size(), 0);
+      for (size_t si = 0; si < e.steps.size(); ++si) {
+        const Step& s2 = e.steps[si];
+        if (s2.kind == StepKind::HashBuild && s2.coord == 0) {
+          CoordTable& t = c0.own_table;
+          const size_t words = hash_capacity_for(n) * 2;
+          if (words <= t.cap * 2 && nj + (t.filter_words ? 2 : 1) <= kMaxFillJobs) {
+            add(t.slots(), words, 0xFFFFFFFFu);
+            if (t.filter_words) add(t.filter.p, t.filter_words, 0u);
+            t.precleared_for = n;
+          }
+        } else if (s2.kind == StepKind::RulebookSparse) {
+          Rulebook& rb = e.rulebooks[s2.rulebook]->rb;
+          if (rb.bitmap.p && rb.bitmap_words && add(rb.bitmap.p, rb.bitmap_words, 0u)) rb.bitmap_precleared = true;
+        } else if (s2.kind == StepKind::Dense) {
+          RtTensor& o = e.tensors[s2.t_out];
+          size_t numel = 1;
+          for (int j = 0; j < 5; ++j) numel *= (size_t)s2.dense_shape[j];
+          if (numel % 2 == 0 && add(o.data, numel / 2, 0u)) e.dense_precleared[si] = 1;
+        }
+      }
+      int rc = fill_multi(jobs, nj, e.in_count.as<uint32_t>(), e.dds, n, stream);
       if (rc) return rc;
       c0.n_dev = e.in_count.as<uint32_t>();
       RtTensor& t = e.tensors[e.inputs[0]];
@@ -891,8 +923,10 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
       const RtTensor& x = e.tensors[st.t_in];
       RtTensor& o = e.tensors[st.t_out];
       const CoordSet& cs = e.coords[x.coord];
+      const size_t si = (size_t)(&st - e.steps.data());
+      const bool pre = si < e.dense_precleared.size() && e.dense_precleared[si];
       return scatter_dense(x.data, x.dtype, x.range, (uint32_t)x.c, x.ld, cs.idx, cs.n_bound, cs.n_dev, st.dense_shape,
-                           st.has_perm ? st.perm : nullptr, o.data, stream);
+                           st.has_perm ? st.perm : nullptr, o.data, stream, pre);
     }
     case StepKind::Permute: {
       const RtTensor& x = e.tensors[st.t_in];

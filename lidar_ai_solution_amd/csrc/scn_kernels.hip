@@ -153,6 +153,43 @@ __global__ void k_fill_u32(uint32_t* __restrict__ p, uint32_t value, size_t coun
   for (size_t j = n4 * 4 + i; j < count; j += stride) p[j] = value;
 }
 
+// Several fills (and the publication of a clamped row count) in one launch: grid.y = job.
+struct FillJobs {
+  FillJob j[kMaxFillJobs];
+};
+
+__global__ __launch_bounds__(256) void k_fill_multi(FillJobs jobs, uint32_t* count_dst, const uint32_t* n_dev,
+                                                    uint32_t n_bound) {
+  if (count_dst && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+    const uint32_t n = eff_n(n_dev, n_bound);
+    count_dst[0] = n;
+    count_dst[1] = n;
+  }
+  const FillJob job = jobs.j[blockIdx.y];
+  uint32_t* p = reinterpret_cast<uint32_t*>(job.p);
+  const size_t stride = (size_t)gridDim.x * 256;
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t n4 = job.count / 4;
+  const uint4 v4 = make_uint4(job.value, job.value, job.value, job.value);
+  for (size_t k = i; k < n4; k += stride) reinterpret_cast<uint4*>(p)[k] = v4;
+  for (size_t k = n4 * 4 + i; k < job.count; k += stride) p[k] = job.value;
+}
+
+int fill_multi(const FillJob* jobs, int n_jobs, uint32_t* count_dst, const uint32_t* n_dev, uint32_t n_bound,
+               hipStream_t stream) {
+  SCN_REQUIRE(n_jobs >= 0 && n_jobs <= kMaxFillJobs, SCN_ERR_INVALID, "fill_multi: too many jobs");
+  FillJobs fj;
+  memset(&fj, 0, sizeof(fj));
+  for (int i = 0; i < n_jobs; ++i) {
+    SCN_REQUIRE(((uintptr_t)jobs[i].p & 15) == 0, SCN_ERR_INVALID, "fill_multi: pointer not 16-byte aligned");
+    fj.j[i] = jobs[i];
+  }
+  hipLaunchKernelGGL(k_fill_multi, dim3(1024, n_jobs > 0 ? n_jobs : 1), dim3(256), 0, stream, fj, count_dst, n_dev,
+                     n_bound);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
 int fill_u32(void* p, uint32_t value, size_t count, hipStream_t stream) {
   if (count == 0) return SCN_OK;
   SCN_REQUIRE(((uintptr_t)p & 15) == 0, SCN_ERR_INVALID, "fill_u32: pointer not 16-byte aligned");
@@ -241,12 +278,16 @@ int hash_build(const CoordTable& t, const int32_t* idx, uint32_t n, const uint32
   SCN_REQUIRE(grid_fits_u32(grid), SCN_ERR_UNSUPPORTED, "grid %dx%dx%d does not fit 32-bit keys", grid[0], grid[1],
               grid[2]);
   const_cast<CoordTable&>(t).mask = (uint32_t)(hash_capacity_for(n) - 1);
-  int rc = fill_u32(t.slots(), 0xFFFFFFFFu, ((size_t)t.mask + 1) * 2, stream);
-  if (rc) return rc;
-  if (t.filter_words) {
-    rc = fill_u32(t.filter.p, 0u, t.filter_words, stream);
+  int rc = SCN_OK;
+  if (t.precleared_for != n) {  // not already cleared (for exactly this size) by the caller's batched fill
+    rc = fill_u32(t.slots(), 0xFFFFFFFFu, ((size_t)t.mask + 1) * 2, stream);
     if (rc) return rc;
+    if (t.filter_words) {
+      rc = fill_u32(t.filter.p, 0u, t.filter_words, stream);
+      if (rc) return rc;
+    }
   }
+  const_cast<CoordTable&>(t).precleared_for = 0xFFFFFFFFu;
   Int3 g{{grid[0], grid[1], grid[2]}};
   const uint32_t blocks = n ? ceil_div(n, 256) : 1;
   hipLaunchKernelGGL(k_hash_insert, dim3(blocks), dim3(256), 0, stream, t.slots(), t.mask,
@@ -302,16 +343,32 @@ __global__ __launch_bounds__(1024) void k_scan_blocksums(uint32_t* vals, uint32_
 // Sparse bitmaps (fewer set bits than words): one thread per word expands its bits in rank order.
 // Optional outputs: coordinate rows and the per-word exclusive prefix (rank of the word's first bit),
 // which together with the bitmap answers "row of this cell" (see coord_row).
-// Block = 1024 threads = 1024 words.
+// Block = 1024 threads = 1024 words.  blockoff holds either the exclusive scan of the per-block counts
+// (raw_sums = 0) or the counts themselves (raw_sums = 1: every block adds up the counts before it, and
+// the last block publishes the totals in counters -- one launch less than a separate scan).
 __global__ __launch_bounds__(1024) void k_bitmap_expand(const uint32_t* __restrict__ bitmap,
                                                         const uint32_t* __restrict__ blockoff, Int3 grid, uint32_t cap,
-                                                        int4* coords_out, uint32_t* prefix_out) {
+                                                        int4* coords_out, uint32_t* prefix_out, int raw_sums,
+                                                        uint32_t* counters) {
   __shared__ uint32_t scratch[17];
   const size_t t = (size_t)blockIdx.x * 1024 + threadIdx.x;
   uint32_t bits = bitmap[t];
   const uint32_t c = __popc(bits);
+  uint32_t base;
+  if (raw_sums) {
+    uint32_t part = 0;
+    for (uint32_t i = threadIdx.x; i < blockIdx.x; i += 1024) part += blockoff[i];
+    (void)block_exclusive_scan(part, scratch, &base);
+  } else {
+    base = blockoff[blockIdx.x];
+  }
   uint32_t total;
-  uint32_t rank = blockoff[blockIdx.x] + block_exclusive_scan(c, scratch, &total);
+  uint32_t rank = base + block_exclusive_scan(c, scratch, &total);
+  if (raw_sums && counters && blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+    const uint32_t all = base + total;
+    counters[1] = all;
+    counters[0] = all < cap ? all : cap;
+  }
   if (prefix_out) prefix_out[t] = rank;
   if (c == 0 || coords_out == nullptr) return;
   const uint32_t g12 = (uint32_t)grid.v[1] * (uint32_t)grid.v[2];
@@ -648,8 +705,11 @@ int Rulebook::build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev
     in_lookup = own_in_table.lookup();
   }
   // occupancy bitmap of the outputs -> ordered unique output coordinates + per-word ranks
-  rc = fill_u32(bitmap.p, 0u, words, stream);
-  if (rc) return rc;
+  if (!bitmap_precleared) {
+    rc = fill_u32(bitmap.p, 0u, words, stream);
+    if (rc) return rc;
+  }
+  bitmap_precleared = false;
   const GeomDev gd = to_dev(geom);
   if (n) {
     hipLaunchKernelGGL(k_mark_outputs, dim3(ceil_div(n, 256)), dim3(256), 0, stream, (const int4*)idx, n_dev, n, gd,
@@ -658,19 +718,22 @@ int Rulebook::build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev
   const uint32_t nblocks = (uint32_t)(words / kWordsPerBlock);
   hipLaunchKernelGGL(k_bitmap_blocksum, dim3(nblocks), dim3(256), 0, stream, bitmap.as<uint32_t>(),
                      blocksum.as<uint32_t>());
-  hipLaunchKernelGGL(k_scan_blocksums, dim3(1), dim3(1024), 0, stream, blocksum.as<uint32_t>(), nblocks, cnt,
-                     n_bound_out);
+  // up to a few thousand blocks every expand block adds up the counts before it itself
+  const int raw = nblocks <= 8192 ? 1 : 0;
+  if (!raw)
+    hipLaunchKernelGGL(k_scan_blocksums, dim3(1), dim3(1024), 0, stream, blocksum.as<uint32_t>(), nblocks, cnt,
+                       n_bound_out);
   const Int3 og{{geom.grid_out[0], geom.grid_out[1], geom.grid_out[2]}};
   const uint64_t cells = (uint64_t)geom.grid_out[0] * geom.grid_out[1] * geom.grid_out[2];
   if (cells <= 32ull * std::max(n_bound_out, 1u)) {
     // dense output grid: per-word ranks, then one thread per cell
     hipLaunchKernelGGL(k_bitmap_expand, dim3(nblocks), dim3(1024), 0, stream, bitmap.as<uint32_t>(),
-                       blocksum.as<uint32_t>(), og, n_bound_out, (int4*)nullptr, prefix.as<uint32_t>());
+                       blocksum.as<uint32_t>(), og, n_bound_out, (int4*)nullptr, prefix.as<uint32_t>(), raw, cnt);
     hipLaunchKernelGGL(k_expand_cells, dim3((unsigned)((cells + 255) / 256)), dim3(256), 0, stream,
                        bitmap.as<uint32_t>(), prefix.as<uint32_t>(), (uint32_t)cells, og, n_bound_out, (int4*)out_idx.p);
   } else {
     hipLaunchKernelGGL(k_bitmap_expand, dim3(nblocks), dim3(1024), 0, stream, bitmap.as<uint32_t>(),
-                       blocksum.as<uint32_t>(), og, n_bound_out, (int4*)out_idx.p, prefix.as<uint32_t>());
+                       blocksum.as<uint32_t>(), og, n_bound_out, (int4*)out_idx.p, prefix.as<uint32_t>(), raw, cnt);
   }
   SCN_HIP(hipGetLastError());
   rc = launch_build_nbr(*this, out_indices, cnt, n_bound_out, false, nullptr, stream);
@@ -1735,7 +1798,8 @@ __global__ __launch_bounds__(256) void k_scatter_dense(const void* feat, int dty
 }
 
 int scatter_dense(const void* feat, int dtype, float range, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
-                  const uint32_t* n_dev, const int dense_shape[5], const int perm[5], void* out, hipStream_t stream) {
+                  const uint32_t* n_dev, const int dense_shape[5], const int perm[5], void* out, hipStream_t stream,
+                  bool precleared) {
   SCN_REQUIRE(out && dense_shape, SCN_ERR_INVALID, "scatter_dense: null pointer");
   const float scale = range > 0.f ? range / 127.f : 1.f;
   SCN_REQUIRE(dense_shape[0] == 1 && (uint32_t)dense_shape[1] == c, SCN_ERR_INVALID,
@@ -1759,8 +1823,10 @@ int scatter_dense(const void* feat, int dtype, float range, uint32_t c, uint32_t
   for (int j = 0; j < 5; ++j) dstride[p[j]] = tstride[j];
   const size_t numel = (size_t)s;
   SCN_REQUIRE(numel % 2 == 0, SCN_ERR_UNSUPPORTED, "scatter_dense: odd element count");
-  int rc = fill_u32(out, 0u, numel / 2, stream);
-  if (rc) return rc;
+  if (!precleared) {
+    int rc = fill_u32(out, 0u, numel / 2, stream);
+    if (rc) return rc;
+  }
   if (n == 0) return SCN_OK;
   SCN_REQUIRE(feat && idx, SCN_ERR_INVALID, "scatter_dense: null input");
   DenseStrides st{dstride[1], dstride[2], dstride[3], dstride[4], dense_shape[2], dense_shape[3], dense_shape[4]};
@@ -2016,7 +2082,7 @@ int scn_voxelizer_forward(scn_voxelizer* v, const void* points_fp16_dev, uint32_
                      (uint32_t)p.max_voxels);
   hipLaunchKernelGGL(k_bitmap_expand, dim3(nblocks), dim3(1024), 0, stream, v->bitmap.as<uint32_t>(),
                      v->blocksum.as<uint32_t>(), Int3{{g.og[0], g.og[1], g.og[2]}}, (uint32_t)p.max_voxels,
-                     (int4*)v->idx.p, v->prefix.as<uint32_t>());
+                     (int4*)v->idx.p, v->prefix.as<uint32_t>(), 0, (uint32_t*)nullptr);
   if (num_points) {
     hipLaunchKernelGGL(k_vox_assign, dim3(ceil_div(num_points, 256)), dim3(256), 0, stream, v->pkey.as<uint32_t>(),
                        num_points, v->bitmap.as<uint32_t>(), v->prefix.as<uint32_t>(), p.max_voxels,

@@ -25,6 +25,7 @@ struct CoordTable {
   uint32_t mask = 0;  // slots in use - 1 (power of two <= cap), set by the last build
   DevBuf filter;             // occupancy bitmap of the grid (optional, see alloc_filter)
   size_t filter_words = 0;
+  uint32_t precleared_for = 0xFFFFFFFFu;  // row count for which slots + filter were cleared by a batched fill
   bool alloc_for(uint32_t max_rows);
   bool alloc_filter(const int grid[3]);
   uint64_t* slots() const { return buf.as<uint64_t>(); }
@@ -63,6 +64,7 @@ struct Rulebook {
   const int32_t* out_indices = nullptr;  // subm: aliases in_indices
   uint32_t n_bound_in = 0, n_bound_out = 0;
   bool built = false;
+  bool bitmap_precleared = false;  // the next build_sparse finds its output bitmap already zeroed
 
   bool init(uint32_t max_in_, uint32_t max_out_, int kvol);
   int reserve_sparse(const int out_grid[3], bool need_own_in_table);
@@ -101,6 +103,15 @@ int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, cons
 
 int set_count(uint32_t* dst, const uint32_t* n_dev, uint32_t n_bound, hipStream_t stream);
 int fill_u32(void* p, uint32_t value, size_t count, hipStream_t stream);
+// several fills and (count_dst != nullptr) the publication of min(*n_dev, n_bound) in one launch
+struct FillJob {
+  void* p;
+  size_t count;  // 32-bit words
+  uint32_t value;
+};
+constexpr int kMaxFillJobs = 12;
+int fill_multi(const FillJob* jobs, int n_jobs, uint32_t* count_dst, const uint32_t* n_dev, uint32_t n_bound,
+               hipStream_t stream);
 int hash_build(const CoordTable& t, const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3],
                uint32_t* n_eff_out, hipStream_t stream);
 int hash_query(const CoordTable& t, const int32_t* coords, uint32_t n, const int grid[3], int32_t* rows,
@@ -114,7 +125,8 @@ int add_relu(const void* a, int a_dtype, float a_range, float a_rq, const void* 
              float b_rq, void* out, int out_dtype, float out_range, int relu, uint32_t c, uint32_t n,
              const uint32_t* n_dev, hipStream_t stream);
 int scatter_dense(const void* feat, int dtype, float range, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
-                  const uint32_t* n_dev, const int dense_shape[5], const int perm[5], void* out, hipStream_t stream);
+                  const uint32_t* n_dev, const int dense_shape[5], const int perm[5], void* out, hipStream_t stream,
+                  bool precleared = false);
 
 int permute_dense(const void* in, const int64_t in_shape[5], const int perm[5], void* out, hipStream_t stream);
 
