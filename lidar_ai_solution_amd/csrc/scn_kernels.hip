@@ -1526,17 +1526,17 @@ static void launch_conv_lds(const ConvArgs& a, hipStream_t stream) {
 // workgroup per CU, so its duration is that of the busiest CU: 257 tiles of 256 rows on 256 CUs take
 // as long as 512.  With the expected row count (the count of the previous forward, see
 // Rulebook::n_out_hint) the tile height is chosen so that all rows fit one workgroup per CU when they
-// can: 8, 10 or 12 waves of 32 rows; beyond 384 rows per CU it is 8 waves and two workgroups per CU.
+// can: 8 to 12 waves of 32 rows; beyond 384 rows per CU it is 8 waves and two workgroups per CU.
 static int conv_lds_waves(uint32_t n_hint) {
   static const int forced = [] {
     const char* e = getenv("SCN_CONV_WAVES");
     return e ? atoi(e) : 0;
   }();
-  if (forced == 8 || forced == 10 || forced == 12) return forced;
+  if (forced >= 8 && forced <= 12) return forced;
   constexpr uint32_t kCus = 256;
-  if (n_hint <= kCus * 256u) return 8;
-  if (n_hint <= kCus * 320u) return 10;
-  if (n_hint <= kCus * 384u) return 12;
+  const uint32_t waves = ceil_div(n_hint, kCus * 32u);  // 32-row tiles per CU
+  if (waves <= 8) return 8;
+  if (waves <= 12) return (int)waves;
   return 8;
 }
 
@@ -1547,7 +1547,9 @@ static bool dispatch_mt32(int mt, uint32_t n_hint, const ConvArgs& a, hipStream_
     case 2: launch_conv_lds<EL, CHUNKS, 2, 8>(a, stream); return true;
     case 4:
       switch (conv_lds_waves(n_hint)) {
+        case 9: launch_conv_lds<EL, CHUNKS, 4, 9>(a, stream); return true;
         case 10: launch_conv_lds<EL, CHUNKS, 4, 10>(a, stream); return true;
+        case 11: launch_conv_lds<EL, CHUNKS, 4, 11>(a, stream); return true;
         case 12: launch_conv_lds<EL, CHUNKS, 4, 12>(a, stream); return true;
         default: launch_conv_lds<EL, CHUNKS, 4, 8>(a, stream); return true;
       }
