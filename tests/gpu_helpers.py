@@ -119,7 +119,9 @@ class GpuConv:
             self.L.scn_conv_destroy(self.h)
             self.h = None
 
-    def forward(self, rb, x_dev, n_out, x_range=127.0, relu=False, out_int8=False, out_range=127.0, want_acc=False, **res):
+    def forward(self, rb, x_dev, n_out, x_range=127.0, relu=False, out_int8=False, out_range=127.0, want_acc=False,
+                out_ld=None, **res):
+        """out_ld: output row stride in elements (default: channels rounded up to 16, what the kernels need)."""
         io = capi.ConvIO()
         io.x_dev = x_dev.data_ptr()
         io.x_ld = x_dev.shape[1]
@@ -127,9 +129,10 @@ class GpuConv:
         io.relu = int(relu)
         io.out_dtype = capi.DTYPE_INT8 if out_int8 else capi.DTYPE_FP16
         io.out_dynamic_range = out_range
-        out = torch.zeros((max(n_out, 1), self.cout), dtype=torch.int8 if out_int8 else torch.float16, device=DEV)
+        ow = out_ld if out_ld is not None else (self.cout + 15) // 16 * 16
+        out = torch.zeros((max(n_out, 1), ow), dtype=torch.int8 if out_int8 else torch.float16, device=DEV)
         io.out_dev = out.data_ptr()
-        io.out_ld = self.cout
+        io.out_ld = ow
         acc = None
         if want_acc:
             acc = torch.zeros((max(n_out, 1), self.cout), dtype=torch.int32 if self.precision == 2 else torch.float32, device=DEV)

@@ -206,6 +206,69 @@ def test_int8_conv_shapes_bit_exact(cin, cout, centerpoint_input):
     assert np.array_equal(out16.cpu().numpy().view(np.uint16), ref16.view(np.uint16))
 
 
+@pytest.mark.parametrize("n", [66000, 75000, 84000, 93000, 101000])
+def test_int8_conv_workgroup_heights(n):
+    """128-channel layers pick their workgroup height (8..12 waves of 32 rows) from the row count of the
+    rulebook's previous build: every height, and the two-workgroups-per-CU case above 98,304 rows, gives
+    the same bit-exact result.  Clustered coordinates so that most offsets have neighbours."""
+    rng = np.random.default_rng(n)
+    grid = (6, 300, 300)
+    idx = synth.uniform_voxels(n, n, grid)
+    note(f"int8 conv 128->128 subm, {n} voxels in {grid} (workgroup height from the row count)")
+    x = rng.integers(-127, 128, (n, 128)).astype(np.int8)
+    w, b, ranges = _weights(rng, 128, (3, 3, 3), 128)
+    x_range, out_range = 3.9, 9.0
+    ref_rb = O.rulebook_subm(idx, grid, (3, 3, 3))
+    wq, s_w = O.quantize_weights(w, ranges)
+    acc_ref = O.conv_int8_acc(x, wq, ref_rb)
+    scale = (np.float32(x_range) / np.float32(127) * s_w).astype(np.float32)
+    rb = GpuRulebook(n, n, 27)
+    d_idx = to_dev(idx)
+    rb.build_subm(d_idx, n, grid, (3, 3, 3))
+    torch.cuda.synchronize()
+    rb.build_subm(d_idx, n, grid, (3, 3, 3))  # the second build finds the first one's row count on the host
+    conv = GpuConv(w, ranges, b, capi.PRECISION_INT8)
+    out, acc = conv.forward(rb, to_dev(x), n, x_range=x_range, relu=True, out_int8=True, out_range=out_range, want_acc=True)
+    assert ref_rb.num_pairs > 3 * n
+    assert np.array_equal(acc.cpu().numpy(), acc_ref)
+    assert np.array_equal(out.cpu().numpy(), O.epilogue(acc_ref, scale, b.astype(np.float32), True, True, out_range))
+
+
+@pytest.mark.parametrize("cin,cout,ks", [(48, 96, (3, 3, 3)), (24, 40, (1, 3, 5)), (64, 32, (2, 2, 2)), (128, 64, (5, 3, 3))])
+def test_int8_conv_padded_channels_and_kernel_shapes(cin, cout, ks, centerpoint_input):
+    """Channel counts that are not powers of two (rows padded to 16-byte chunks, partial MFMA tiles), output
+    rows that are not a multiple of 16 bytes (scalar store path), even and large kernel volumes."""
+    _, idx_all = centerpoint_input
+    rng = np.random.default_rng(cin * 100 + cout)
+    idx = idx_all[:9000]
+    n = idx.shape[0]
+    grid = (41, 1440, 1440)
+    kvol = ks[0] * ks[1] * ks[2]
+    note(f"int8 conv {cin}->{cout} k={ks} on {n} fixture voxels")
+    cpad = {48: 64, 24: 32}.get(cin, cin)  # the kernel's row stride: chunks per row rounded to a power of two
+    x = np.zeros((n, cpad), np.int8)
+    x[:, :cin] = rng.integers(-127, 128, (n, cin))
+    w, b, ranges = _weights(rng, cout, ks, cin)
+    x_range, out_range = 3.9, 5.5
+    ref_rb = O.rulebook_subm(idx, grid, ks)
+    wq, s_w = O.quantize_weights(w, ranges)
+    acc_ref = O.conv_int8_acc(np.ascontiguousarray(x[:, :cin]), wq, ref_rb)
+    scale = (np.float32(x_range) / np.float32(127) * s_w).astype(np.float32)
+    rb = GpuRulebook(n, n, kvol)
+    rb.build_subm(to_dev(idx), n, grid, ks)
+    conv = GpuConv(w, ranges, b, capi.PRECISION_INT8)
+    want_acc = cout % 16 == 0
+    out, acc = conv.forward(rb, to_dev(x), n, x_range=x_range, relu=True, out_int8=True, out_range=out_range, want_acc=want_acc)
+    if want_acc:
+        assert np.array_equal(acc.cpu().numpy(), acc_ref)
+    ref = O.epilogue(acc_ref, scale, b.astype(np.float32), True, True, out_range)
+    assert np.array_equal(out.cpu().numpy()[:, :cout], ref)
+    # a row stride that is not a multiple of 16 bytes takes the 4-byte store path
+    out2, _ = conv.forward(rb, to_dev(x), n, x_range=x_range, relu=True, out_int8=True, out_range=out_range,
+                           out_ld=(cout + 15) // 16 * 16 + 4)
+    assert np.array_equal(out2.cpu().numpy()[:, :cout], ref)
+
+
 @pytest.mark.parametrize("cin,cout", [(5, 16), (16, 16), (32, 64), (128, 128)])
 def test_fp16_conv_within_tolerance(cin, cout, centerpoint_input):
     """fp16 MFMA path: fp32 accumulation in hardware order.  Tolerance (stated): every accumulator
