@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--points", type=int, default=250000)
     ap.add_argument("--no-graph", action="store_true", help="launch kernels directly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-reps", type=int, default=3)
+    ap.add_argument("--cpu-reps", type=int, default=5)
     ap.add_argument("--layers", action="store_true", help="also print the per-step table to stderr")
     ap.add_argument("--copy-probe", action="store_true",
                     help="first launch a plain copy kernel of known size (k_convert_rows fp16->fp16, 512 MiB read + "
