@@ -191,11 +191,23 @@ struct scn_engine {
   int alloc_grid[3] = {0, 0, 0};
   bool profiling = false;
   bool input_set = false;
+  // SCN_BUILD_AUX_STREAM: hash and rulebook construction depend on coordinates only, so they run on a
+  // second stream ahead of the convolutions; a convolution waits for its rulebook's event.
+  hipStream_t aux = nullptr;
+  hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+  std::vector<hipEvent_t> rb_ready;   // per rulebook
+  std::vector<int> rb_seq;            // per rulebook: position in the auxiliary stream's order (this forward)
+  std::vector<int> coord_rb;          // per coordinate set: rulebook that produced it (-1: graph input)
   ~scn_engine() {
     for (auto& s : steps) {
       if (s.ev0) (void)hipEventDestroy(s.ev0);
       if (s.ev1) (void)hipEventDestroy(s.ev1);
     }
+    for (auto ev : rb_ready)
+      if (ev) (void)hipEventDestroy(ev);
+    if (ev_fork) (void)hipEventDestroy(ev_fork);
+    if (ev_join) (void)hipEventDestroy(ev_join);
+    if (aux) (void)hipStreamDestroy(aux);
   }
 };
 
@@ -780,6 +792,13 @@ static int allocate_runtime(scn_engine& e) {
         const size_t bytes = (size_t)e.coords[o.coord].cap * o.ld * 4;
         if (o.acc.bytes < bytes && !o.acc.alloc(bytes)) return SCN_ERR_HIP;
       }
+  }
+  if ((e.flags & SCN_BUILD_AUX_STREAM) && !e.aux) {
+    SCN_HIP(hipStreamCreateWithFlags(&e.aux, hipStreamNonBlocking));  // default priority
+    SCN_HIP(hipEventCreateWithFlags(&e.ev_fork, hipEventDisableTiming));
+    SCN_HIP(hipEventCreateWithFlags(&e.ev_join, hipEventDisableTiming));
+    e.rb_ready.assign(e.rulebooks.size(), nullptr);
+    for (auto& ev : e.rb_ready) SCN_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
   }
   memcpy(e.alloc_grid, e.in_grid, 12);
   e.allocated = true;
@@ -1519,6 +1538,14 @@ int scn_engine_forward(scn_engine* e, void* stream_) {
     int rc = allocate_runtime(*e);
     if (rc) return rc;
   }
+  // Two streams unless per-step profiling is on.  The auxiliary stream is in order, so waiting for a
+  // rulebook's event also covers everything built before it.
+  const bool dual = e->aux != nullptr && !e->profiling;
+  int aux_seq = 0, waited_seq = 0;
+  if (dual) {
+    e->rb_seq.assign(e->rulebooks.size(), 0);
+    e->coord_rb.assign(e->coords.size(), -1);
+  }
   for (auto& st : e->steps) {
     if (e->profiling) {
       if (!st.ev0) {
@@ -1527,12 +1554,44 @@ int scn_engine_forward(scn_engine* e, void* stream_) {
       }
       SCN_HIP(hipEventRecord(st.ev0, stream));
     }
-    int rc = run_step(*e, st, stream);
+    const bool coord_step =
+        st.kind == StepKind::HashBuild || st.kind == StepKind::RulebookSubm || st.kind == StepKind::RulebookSparse;
+    hipStream_t run_on = stream;
+    if (dual && coord_step) {
+      run_on = e->aux;
+    } else if (dual && st.kind != StepKind::InputCount) {
+      // rulebook this step depends on: its own (convolutions) or the one that produced its rows
+      int rb = -1;
+      if (st.kind == StepKind::Conv) {
+        rb = st.rulebook;
+      } else if (st.t_in >= 0 && st.t_in < (int)e->tensors.size()) {
+        const int c = e->tensors[st.t_in].coord;
+        if (c >= 0 && c < (int)e->coord_rb.size()) rb = e->coord_rb[c];
+      }
+      if (rb >= 0 && e->rb_seq[rb] > waited_seq) {
+        SCN_HIP(hipStreamWaitEvent(stream, e->rb_ready[rb], 0));
+        waited_seq = e->rb_seq[rb];
+      }
+    }
+    int rc = run_step(*e, st, run_on);
     if (rc) {
       SCN_LOGE("forward failed at step %s", st.label.c_str());
       return rc;
     }
+    if (dual && st.kind == StepKind::InputCount) {
+      SCN_HIP(hipEventRecord(e->ev_fork, stream));
+      SCN_HIP(hipStreamWaitEvent(e->aux, e->ev_fork, 0));
+    }
+    if (dual && (st.kind == StepKind::RulebookSubm || st.kind == StepKind::RulebookSparse)) {
+      SCN_HIP(hipEventRecord(e->rb_ready[st.rulebook], e->aux));
+      e->rb_seq[st.rulebook] = ++aux_seq;
+      if (st.kind == StepKind::RulebookSparse) e->coord_rb[e->rulebooks[st.rulebook]->coord_out] = st.rulebook;
+    }
     if (e->profiling) SCN_HIP(hipEventRecord(st.ev1, stream));
+  }
+  if (dual) {
+    SCN_HIP(hipEventRecord(e->ev_join, e->aux));
+    SCN_HIP(hipStreamWaitEvent(stream, e->ev_join, 0));
   }
   if (e->profiling) {
     SCN_HIP(hipStreamSynchronize(stream));

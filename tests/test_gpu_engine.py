@@ -150,6 +150,49 @@ def test_int8_backbone_every_layer_bit_exact(cp_models, centerpoint_input):
     assert np.count_nonzero(got) > 100000
 
 
+def test_auxiliary_stream_gives_identical_results(cp_models, centerpoint_input):
+    """with_auxiliary_stream: rulebooks are built on the engine's second stream, convolutions wait for
+    their rulebook's event.  Outputs must equal the single-stream engine's bit for bit -- on direct
+    launches with inputs of changing size, and on replays of a captured HIP graph (several replays
+    with eager work and synchronisations in between, each checked)."""
+    feats, idx = centerpoint_input
+    _, g8 = cp_models
+    note("int8 backbone, auxiliary stream vs single stream")
+    ref_eng = Engine.from_graph(g8, "int8")
+    aux_eng = Engine.from_graph(g8, "int8", with_auxiliary_stream=True)
+    st = torch.cuda.Stream()
+    keep = []
+    for n in (feats.shape[0], 30000, 61234, feats.shape[0]):
+        f, i = to_dev(feats[:n]), to_dev(idx[:n])
+        keep.append((f, i))
+        ref_eng.set_input(f, i, GRID_ZYX)
+        ref_eng.forward()
+        torch.cuda.synchronize()
+        want = ref_eng.output(0).torch().cpu().numpy().view(np.uint16)
+        aux_eng.set_input(f, i, GRID_ZYX)
+        with torch.cuda.stream(st):
+            aux_eng.forward()
+            aux_eng.forward()  # back to back: the second forward's clears must wait for the first one's joins
+        torch.cuda.synchronize()
+        got = aux_eng.output(0).torch().cpu().numpy().view(np.uint16)
+        assert np.array_equal(got, want), f"direct launches, n={n}"
+    note("captured graph of the two-stream forward, 4 replays")
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(st):
+        aux_eng.forward()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(g, stream=st):
+        aux_eng.forward()
+    torch.cuda.synchronize()
+    for rep in range(4):
+        scratch = torch.randn(1 << 20, device=DEV).sum().item()  # eager work between replays
+        assert np.isfinite(scratch)
+        g.replay()
+        torch.cuda.synchronize()
+        got = aux_eng.output(0).torch().cpu().numpy().view(np.uint16)
+        assert np.array_equal(got, want), f"replay {rep}"
+
+
 def _fp16_region_override(graph, eng):
     """Outputs of fp16-computed convolutions (the only nodes whose result depends on the MFMA summation
     order), read back from the keep-all engine: name -> array.  Add / Relu are deterministic given
