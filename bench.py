@@ -255,6 +255,13 @@ def main():
         for _ in range(args.warmup):
             step()
     torch.cuda.synchronize()
+    # host time to enqueue one forward (must stay below the GPU time per step for the loop to be GPU bound)
+    e0 = time.perf_counter()
+    with torch.cuda.stream(stream):
+        for _ in range(10):
+            step()
+    enqueue_ms = (time.perf_counter() - e0) / 10 * 1e3
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
     with torch.cuda.stream(stream):
         for _ in range(args.steps):
@@ -367,6 +374,7 @@ def main():
                    "auxiliary_stream": not args.no_aux_stream, "output": out_view.shape},
         "voxels_per_s": round(nvox * 1e3 / ms_per_step, 1),
         "voxelization_ms": round(vox_ms, 4),
+        "host_enqueue_ms_per_step": round(enqueue_ms, 4),
         "backbone_gop_per_frame": round(total_ops / 1e9, 2),
         "backbone_algorithmic_MB_per_frame": round(total_bytes / 1e6, 1),
         "whole_backbone_TOPs": round(total_ops / (ms_per_step * 1e-3) / 1e12, 3),
