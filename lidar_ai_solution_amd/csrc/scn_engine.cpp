@@ -177,7 +177,10 @@ struct scn_engine {
   std::vector<std::unique_ptr<RbSlot>> rulebooks;
   std::vector<std::unique_ptr<ConvWeights>> convs;
   std::vector<Step> steps;
-  std::vector<char> dense_precleared;  // per step: its dense output was zeroed by the forward's batched fill
+  std::vector<char> dense_precleared;  // per step: the forward's batched fill zeroed its dense output (1) or reset its row map (2)
+  bool dense_map_built = false;        // the step about to run had its row map built on the auxiliary stream
+  hipEvent_t ev_map = nullptr;
+  std::vector<DevBuf> dense_maps;      // per step: cell -> row map of a ScatterDense whose layout allows the dense-major pass
   std::map<std::string, int> tensor_by_name;
   // input binding
   const void* in_feat = nullptr;
@@ -207,6 +210,7 @@ struct scn_engine {
       if (ev) (void)hipEventDestroy(ev);
     if (ev_fork) (void)hipEventDestroy(ev_fork);
     if (ev_join) (void)hipEventDestroy(ev_join);
+    if (ev_map) (void)hipEventDestroy(ev_map);
     if (aux) (void)hipStreamDestroy(aux);
   }
 };
@@ -785,6 +789,13 @@ static int allocate_runtime(scn_engine& e) {
   }
   for (auto& x : e.tensors)
     if (x.dense && x.view_of >= 0) x.data = e.tensors[x.view_of].data;
+  e.dense_maps.resize(e.steps.size());
+  for (size_t si = 0; si < e.steps.size(); ++si) {
+    const Step& st = e.steps[si];
+    if (st.kind != StepKind::Dense) continue;
+    const size_t cells = scatter_dense_map_cells(st.dense_shape, st.has_perm ? st.perm : nullptr);
+    if (cells && e.dense_maps[si].bytes < cells * 4 && !e.dense_maps[si].alloc(cells * 4)) return SCN_ERR_HIP;
+  }
   if (keep_all) {
     for (auto& st : e.steps)
       if (st.kind == StepKind::Conv) {
@@ -797,6 +808,7 @@ static int allocate_runtime(scn_engine& e) {
     SCN_HIP(hipStreamCreateWithFlags(&e.aux, hipStreamNonBlocking));  // default priority
     SCN_HIP(hipEventCreateWithFlags(&e.ev_fork, hipEventDisableTiming));
     SCN_HIP(hipEventCreateWithFlags(&e.ev_join, hipEventDisableTiming));
+    SCN_HIP(hipEventCreateWithFlags(&e.ev_map, hipEventDisableTiming));
     e.rb_ready.assign(e.rulebooks.size(), nullptr);
     for (auto& ev : e.rb_ready) SCN_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
   }
@@ -845,7 +857,11 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
           RtTensor& o = e.tensors[s2.t_out];
           size_t numel = 1;
           for (int j = 0; j < 5; ++j) numel *= (size_t)s2.dense_shape[j];
-          if (numel % 2 == 0 && add(o.data, numel / 2, 0u)) e.dense_precleared[si] = 1;
+          if (si < e.dense_maps.size() && e.dense_maps[si].p) {
+            if (add(e.dense_maps[si].p, e.dense_maps[si].bytes / 4, 0xFFFFFFFFu)) e.dense_precleared[si] = 2;
+          } else if (numel % 2 == 0 && add(o.data, numel / 2, 0u)) {
+            e.dense_precleared[si] = 1;
+          }
         }
       }
       int rc = fill_multi(jobs, nj, e.in_count.as<uint32_t>(), e.dds, n, stream);
@@ -943,9 +959,10 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
       RtTensor& o = e.tensors[st.t_out];
       const CoordSet& cs = e.coords[x.coord];
       const size_t si = (size_t)(&st - e.steps.data());
-      const bool pre = si < e.dense_precleared.size() && e.dense_precleared[si];
+      const int pre = si < e.dense_precleared.size() ? e.dense_precleared[si] : 0;
+      int32_t* map = si < e.dense_maps.size() ? e.dense_maps[si].as<int32_t>() : nullptr;
       return scatter_dense(x.data, x.dtype, x.range, (uint32_t)x.c, x.ld, cs.idx, cs.n_bound, cs.n_dev, st.dense_shape,
-                           st.has_perm ? st.perm : nullptr, o.data, stream, pre);
+                           st.has_perm ? st.perm : nullptr, o.data, stream, pre == 1, map, pre == 2, e.dense_map_built);
     }
     case StepKind::Permute: {
       const RtTensor& x = e.tensors[st.t_in];
@@ -1573,7 +1590,22 @@ int scn_engine_forward(scn_engine* e, void* stream_) {
         waited_seq = e->rb_seq[rb];
       }
     }
+    if (dual && st.kind == StepKind::Dense) {
+      // The row map needs only the coordinates, which the auxiliary stream has produced (or which came
+      // with the input): build it there, ahead of the convolutions the main stream is still running.
+      const size_t si = (size_t)(&st - e->steps.data());
+      if (si < e->dense_maps.size() && e->dense_maps[si].p && e->dense_precleared[si] == 2) {
+        const CoordSet& cs = e->coords[e->tensors[st.t_in].coord];
+        int rc = scatter_dense_build_map(cs.idx, cs.n_bound, cs.n_dev, st.dense_shape, st.has_perm ? st.perm : nullptr,
+                                         e->dense_maps[si].as<int32_t>(), true, e->aux);
+        if (rc) return rc;
+        SCN_HIP(hipEventRecord(e->ev_map, e->aux));
+        SCN_HIP(hipStreamWaitEvent(stream, e->ev_map, 0));
+        e->dense_map_built = true;
+      }
+    }
     int rc = run_step(*e, st, run_on);
+    e->dense_map_built = false;
     if (rc) {
       SCN_LOGE("forward failed at step %s", st.label.c_str());
       return rc;

@@ -1799,18 +1799,82 @@ __global__ __launch_bounds__(256) void k_scatter_dense(const void* feat, int dty
     if (c0 + j < c_total) dst[(c0 + j) * st.sc] = (_Float16)v[j];
 }
 
-int scatter_dense(const void* feat, int dtype, float range, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
-                  const uint32_t* n_dev, const int dense_shape[5], const int perm[5], void* out, hipStream_t stream,
-                  bool precleared) {
-  SCN_REQUIRE(out && dense_shape, SCN_ERR_INVALID, "scatter_dense: null pointer");
-  const float scale = range > 0.f ? range / 127.f : 1.f;
-  SCN_REQUIRE(dense_shape[0] == 1 && (uint32_t)dense_shape[1] == c, SCN_ERR_INVALID,
-              "scatter_dense: output_shape must be [1, C=%u, D0, D1, D2]", c);
+// Dense-major variant for layouts whose channel axis is outermost (the reference's
+// [1, C, D0, D1, D2] after its Transpose): cell_map[cell] holds the row that occupies a cell or -1,
+// where "cell" is the element offset inside one channel plane.  Pass 1 writes the row numbers,
+// pass 2 walks the dense tensor in memory order and writes every element exactly once (value or
+// zero) in whole 16-byte vectors, so the tensor needs no clear and no partial-line stores.
+__global__ __launch_bounds__(256) void k_cell_map(const int4* __restrict__ coords, uint32_t n_bound,
+                                                  const uint32_t* n_dev, DenseStrides st, int32_t* cell_map) {
+  const uint32_t n = eff_n(n_dev, n_bound);
+  const uint32_t row = blockIdx.x * 256 + threadIdx.x;
+  if (row >= n) return;
+  const int4 p = coords[row];
+  if (p.x != 0 || p.y < 0 || p.y >= st.d0 || p.z < 0 || p.z >= st.d1 || p.w < 0 || p.w >= st.d2) return;
+  cell_map[p.y * st.s0 + p.z * st.s1 + p.w * st.s2] = (int32_t)row;
+}
+
+// One thread per (8 consecutive cells, 8 channels): 8 map entries, up to 8 gathered 8-channel
+// vectors, transposed in registers into 8 stores of 16 bytes (one per channel plane); consecutive
+// lanes own consecutive cell groups, so every store instruction of a wave writes 1 KiB contiguously.
+__global__ __launch_bounds__(128) void k_dense_from_map(const void* feat, int dtype, float scale, uint32_t c_total,
+                                                        uint32_t ld, const int32_t* __restrict__ cell_map,
+                                                        uint32_t cell_groups, uint32_t plane, _Float16* out) {
+  typedef _Float16 v8hh __attribute__((ext_vector_type(8)));
+  const uint32_t g = blockIdx.x * 128 + threadIdx.x;
+  if (g >= cell_groups) return;
+  const uint32_t c0 = blockIdx.y * 8;
+  const int4 ma = *reinterpret_cast<const int4*>(cell_map + (size_t)g * 8);
+  const int4 mb = *reinterpret_cast<const int4*>(cell_map + (size_t)g * 8 + 4);
+  const int m[8] = {ma.x, ma.y, ma.z, ma.w, mb.x, mb.y, mb.z, mb.w};
+  v8hh o[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) o[j] = v8hh{0, 0, 0, 0, 0, 0, 0, 0};
+  if ((ma.x & ma.y & ma.z & ma.w & mb.x & mb.y & mb.z & mb.w) >= 0) {   // some entry is a row
+    // all eight gathers are issued before the first is used; empty cells read row 0 and are masked
+    const bool full = c0 + 8 <= c_total && (ld & 7) == 0;
+    size_t base[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) base[i] = (size_t)(m[i] < 0 ? 0 : m[i]) * ld + c0;
+    if (full && dtype == SCN_DTYPE_FP16) {
+      v8hh h[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) h[i] = *reinterpret_cast<const v8hh*>(reinterpret_cast<const _Float16*>(feat) + base[i]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j][i] = m[i] < 0 ? (_Float16)0 : h[i][j];
+    } else if (full && dtype == SCN_DTYPE_INT8) {
+      typedef signed char v8c __attribute__((ext_vector_type(8)));
+      v8c q[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) q[i] = *reinterpret_cast<const v8c*>(reinterpret_cast<const signed char*>(feat) + base[i]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j][i] = m[i] < 0 ? (_Float16)0 : (_Float16)((float)q[i][j] * scale);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (m[i] < 0) continue;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (c0 + j < c_total) o[j][i] = (_Float16)load_value(feat, dtype, base[i] + j, scale, 0.f, 0.f);
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    if (c0 + j < c_total) *reinterpret_cast<v8hh*>(out + (size_t)(c0 + j) * plane + (size_t)g * 8) = o[j];
+}
+
+// strides (in elements) of dense_shape's five axes inside the (possibly transposed) output
+static bool dense_layout(const int dense_shape[5], const int perm[5], int64_t dstride[5], size_t* numel) {
   int p[5] = {0, 1, 2, 3, 4};
   if (perm) {
     bool seen[5] = {false, false, false, false, false};
     for (int j = 0; j < 5; ++j) {
-      SCN_REQUIRE(perm[j] >= 0 && perm[j] < 5 && !seen[perm[j]], SCN_ERR_INVALID, "scatter_dense: bad permutation");
+      if (perm[j] < 0 || perm[j] >= 5 || seen[perm[j]]) return false;
       seen[perm[j]] = true;
       p[j] = perm[j];
     }
@@ -1821,17 +1885,70 @@ int scatter_dense(const void* feat, int dtype, float range, uint32_t c, uint32_t
     tstride[j] = s;
     s *= dense_shape[p[j]];
   }
-  int64_t dstride[5];
   for (int j = 0; j < 5; ++j) dstride[p[j]] = tstride[j];
-  const size_t numel = (size_t)s;
+  *numel = (size_t)s;
+  return true;
+}
+
+size_t scatter_dense_map_cells(const int dense_shape[5], const int perm[5]) {
+  int64_t dstride[5];
+  size_t numel = 0;
+  if (!dense_shape || dense_shape[0] != 1 || !dense_layout(dense_shape, perm, dstride, &numel)) return 0;
+  const size_t plane = (size_t)dense_shape[2] * dense_shape[3] * dense_shape[4];
+  if (plane == 0 || plane % 8 != 0 || plane > 0x7fffffffu) return 0;
+  return dstride[1] == (int64_t)plane ? plane : 0;   // channel axis outermost
+}
+
+int scatter_dense_build_map(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int dense_shape[5],
+                            const int perm[5], int32_t* cell_map, bool map_precleared, hipStream_t stream) {
+  const size_t plane = scatter_dense_map_cells(dense_shape, perm);
+  SCN_REQUIRE(plane && cell_map, SCN_ERR_INVALID, "scatter_dense: this layout takes no row map");
+  SCN_REQUIRE(n == 0 || idx, SCN_ERR_INVALID, "scatter_dense: null input");
+  int64_t dstride[5];
+  size_t numel = 0;
+  dense_layout(dense_shape, perm, dstride, &numel);
+  DenseStrides st{dstride[1], dstride[2], dstride[3], dstride[4], dense_shape[2], dense_shape[3], dense_shape[4]};
+  if (!map_precleared) {
+    int rc = fill_u32(cell_map, 0xFFFFFFFFu, plane, stream);
+    if (rc) return rc;
+  }
+  if (n)
+    hipLaunchKernelGGL(k_cell_map, dim3(ceil_div(n, 256)), dim3(256), 0, stream, (const int4*)idx, n, n_dev, st, cell_map);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
+int scatter_dense(const void* feat, int dtype, float range, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
+                  const uint32_t* n_dev, const int dense_shape[5], const int perm[5], void* out, hipStream_t stream,
+                  bool precleared, int32_t* cell_map, bool map_precleared, bool map_built) {
+  SCN_REQUIRE(out && dense_shape, SCN_ERR_INVALID, "scatter_dense: null pointer");
+  const float scale = range > 0.f ? range / 127.f : 1.f;
+  SCN_REQUIRE(dense_shape[0] == 1 && (uint32_t)dense_shape[1] == c, SCN_ERR_INVALID,
+              "scatter_dense: output_shape must be [1, C=%u, D0, D1, D2]", c);
+  int64_t dstride[5];
+  size_t numel = 0;
+  SCN_REQUIRE(dense_layout(dense_shape, perm, dstride, &numel), SCN_ERR_INVALID, "scatter_dense: bad permutation");
   SCN_REQUIRE(numel % 2 == 0, SCN_ERR_UNSUPPORTED, "scatter_dense: odd element count");
+  DenseStrides st{dstride[1], dstride[2], dstride[3], dstride[4], dense_shape[2], dense_shape[3], dense_shape[4]};
+  const size_t plane = cell_map ? scatter_dense_map_cells(dense_shape, perm) : 0;
+  if (plane) {
+    SCN_REQUIRE(n == 0 || (feat && idx), SCN_ERR_INVALID, "scatter_dense: null input");
+    if (!map_built) {
+      int rc = scatter_dense_build_map(idx, n, n_dev, dense_shape, perm, cell_map, map_precleared, stream);
+      if (rc) return rc;
+    }
+    const uint32_t groups = (uint32_t)(plane / 8);
+    hipLaunchKernelGGL(k_dense_from_map, dim3(ceil_div(groups, 128), ceil_div(c, 8)), dim3(128), 0, stream, feat, dtype,
+                       scale, c, ld, cell_map, groups, (uint32_t)plane, (_Float16*)out);
+    SCN_HIP(hipGetLastError());
+    return SCN_OK;
+  }
   if (!precleared) {
     int rc = fill_u32(out, 0u, numel / 2, stream);
     if (rc) return rc;
   }
   if (n == 0) return SCN_OK;
   SCN_REQUIRE(feat && idx, SCN_ERR_INVALID, "scatter_dense: null input");
-  DenseStrides st{dstride[1], dstride[2], dstride[3], dstride[4], dense_shape[2], dense_shape[3], dense_shape[4]};
   hipLaunchKernelGGL(k_scatter_dense, dim3(ceil_div(n, 256), ceil_div(c, 8)), dim3(256), 0, stream, feat, dtype, scale, c,
                      ld, (const int4*)idx, n, n_dev, st, (_Float16*)out);
   SCN_HIP(hipGetLastError());
@@ -2216,6 +2333,17 @@ int scn_scatter_dense(const void* feat_dev, int dtype, float dynamic_range, uint
                       const int perm[5], void* out_fp16_dev, void* stream) {
   return scatter_dense(feat_dev, dtype, dynamic_range, c, ld, indices_dev, n, n_dev, dense_shape, perm, out_fp16_dev,
                        (hipStream_t)stream);
+}
+
+size_t scn_scatter_dense_map_cells(const int dense_shape[5], const int perm[5]) {
+  return scatter_dense_map_cells(dense_shape, perm);
+}
+
+int scn_scatter_dense_with_map(const void* feat_dev, int dtype, float dynamic_range, uint32_t c, uint32_t ld,
+                               const int32_t* indices_dev, uint32_t n, const uint32_t* n_dev, const int dense_shape[5],
+                               const int perm[5], void* out_fp16_dev, int32_t* cell_map_dev, void* stream) {
+  return scatter_dense(feat_dev, dtype, dynamic_range, c, ld, indices_dev, n, n_dev, dense_shape, perm, out_fp16_dev,
+                       (hipStream_t)stream, false, cell_map_dev, false);
 }
 
 }  // extern "C"

@@ -126,7 +126,15 @@ int add_relu(const void* a, int a_dtype, float a_range, float a_rq, const void* 
              const uint32_t* n_dev, hipStream_t stream);
 int scatter_dense(const void* feat, int dtype, float range, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
                   const uint32_t* n_dev, const int dense_shape[5], const int perm[5], void* out, hipStream_t stream,
-                  bool precleared = false);
+                  bool precleared = false, int32_t* cell_map = nullptr, bool map_precleared = false,
+                  bool map_built = false);
+// first half of the map variant on its own (it needs only the coordinates): scatter_dense(..., map_built = true)
+// may then follow on another stream once this one is done
+int scatter_dense_build_map(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int dense_shape[5],
+                            const int perm[5], int32_t* cell_map, bool map_precleared, hipStream_t stream);
+// Cells of the row map that lets scatter_dense write the dense tensor in memory order (no clear, whole
+// 16-byte stores); 0 when the layout does not qualify (channel axis not outermost, plane not a multiple of 8).
+size_t scatter_dense_map_cells(const int dense_shape[5], const int perm[5]);
 
 int permute_dense(const void* in, const int64_t in_shape[5], const int perm[5], void* out, hipStream_t stream);
 

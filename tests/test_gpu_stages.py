@@ -413,6 +413,53 @@ def test_convert_add_and_dense():
     assert np.array_equal(out.cpu().numpy().view(np.uint16), O.scatter_dense(O.dequantize(qf, 6.35), idx, dims).view(np.uint16))
 
 
+def test_scatter_dense_with_row_map():
+    """The dense-major variant (row map, no clear, whole 16-byte stores) against the oracle: fp16 and int8
+    rows, channel counts that are not a multiple of 8, permuted spatial axes, a device-side row count, a
+    map holding stale entries, and layouts that do not qualify (channel-last, odd plane)."""
+    L = capi.lib()
+    rng = np.random.default_rng(77)
+    for dims, c, ld, n, perm in [((2, 44, 36), 16, 16, 1500, None), ((2, 44, 36), 16, 16, 1500, (0, 1, 4, 2, 3)),
+                                 ((3, 40, 40), 20, 24, 2500, (0, 1, 2, 3, 4)), ((1, 64, 72), 128, 128, 4000, (0, 1, 3, 2, 4)),
+                                 ((2, 44, 36), 16, 16, 1500, (0, 2, 3, 4, 1)), ((2, 45, 37), 16, 16, 1500, None),
+                                 ((2, 44, 36), 16, 16, 0, None)]:
+        note(f"scatter with map dims={dims} c={c} ld={ld} n={n} perm={perm}")
+        cells = int(np.prod(dims))
+        lin = rng.choice(cells, max(n, 1), replace=False)[:n]
+        idx = np.zeros((n, 4), np.int32)
+        idx[:, 3] = lin % dims[2]; idx[:, 2] = (lin // dims[2]) % dims[1]; idx[:, 1] = lin // (dims[2] * dims[1])
+        shape = capi.i5(1, c, *dims)
+        pm = capi.i5(*perm) if perm else None
+        want_cells = L.scn_scatter_dense_map_cells(shape, pm)
+        qualifies = cells % 8 == 0 and (perm is None or perm[1] == 1)
+        assert want_cells == (cells if qualifies else 0)
+        cell_map = torch.full((max(want_cells, 1),), 5, dtype=torch.int32, device=DEV)   # stale contents
+        oshape = (1, c, *dims) if not perm else tuple((1, c, *dims)[a] for a in perm)
+        for dtype in (capi.DTYPE_FP16, capi.DTYPE_INT8):
+            if dtype == capi.DTYPE_FP16:
+                feat = rng.standard_normal((n, ld)).astype(np.float16); ref_rows = feat[:, :c]; rng_ = 0.0
+            else:
+                feat = rng.integers(-127, 128, (n, ld)).astype(np.int8); ref_rows = O.dequantize(feat[:, :c], 6.35); rng_ = 6.35
+            ref = O.scatter_dense(ref_rows, idx, dims)
+            if perm: ref = np.ascontiguousarray(ref.transpose(perm))
+            out = torch.full(oshape, 3, dtype=torch.float16, device=DEV)
+            d_feat, d_idx = to_dev(feat), to_dev(idx)
+            capi.check(L.scn_scatter_dense_with_map(ptr(d_feat) if n else None, dtype, rng_, c, ld, ptr(d_idx) if n else None,
+                                                    n, None, shape, pm, ptr(out), ptr(cell_map) if want_cells else None, stream()))
+            torch.cuda.synchronize()
+            assert np.array_equal(out.cpu().numpy().view(np.uint16), ref.view(np.uint16))
+            if n:  # device-side count: only the first rows are scattered
+                k = n // 3
+                cnt = to_dev(np.array([k], np.uint32))
+                ref = O.scatter_dense(ref_rows[:k], idx[:k], dims)
+                if perm: ref = np.ascontiguousarray(ref.transpose(perm))
+                out.fill_(7)
+                capi.check(L.scn_scatter_dense_with_map(ptr(d_feat), dtype, rng_, c, ld, ptr(d_idx), n, ptr(cnt), shape, pm,
+                                                        ptr(out), ptr(cell_map) if want_cells else None, stream()))
+                torch.cuda.synchronize()
+                assert np.array_equal(out.cpu().numpy().view(np.uint16), ref.view(np.uint16))
+
+
 # ----------------------------------------------------------------------------- voxelization
 def _voxelizer(max_voxels=160000, max_points=300000):
     p = capi.VoxelizationParam()
