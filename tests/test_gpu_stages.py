@@ -234,7 +234,8 @@ def test_int8_conv_workgroup_heights(n):
     assert np.array_equal(out.cpu().numpy(), O.epilogue(acc_ref, scale, b.astype(np.float32), True, True, out_range))
 
 
-@pytest.mark.parametrize("cin,cout,ks", [(48, 96, (3, 3, 3)), (24, 40, (1, 3, 5)), (64, 32, (2, 2, 2)), (128, 64, (5, 3, 3))])
+@pytest.mark.parametrize("cin,cout,ks", [(48, 96, (3, 3, 3)), (24, 40, (1, 3, 5)), (64, 32, (2, 2, 2)), (128, 64, (5, 3, 3)),
+                                         (64, 64, (2, 2, 2)), (128, 128, (3, 1, 1)), (64, 128, (3, 3, 3)), (128, 128, (1, 1, 2))])
 def test_int8_conv_padded_channels_and_kernel_shapes(cin, cout, ks, centerpoint_input):
     """Channel counts that are not powers of two (rows padded to 16-byte chunks, partial MFMA tiles), output
     rows that are not a multiple of 16 bytes (scalar store path), even and large kernel volumes."""
