@@ -51,6 +51,7 @@ struct NodeDesc {
   int ks[3] = {1, 1, 1}, stride[3] = {1, 1, 1}, pad[3] = {0, 0, 0}, dil[3] = {1, 1, 1};
   float in_range = 0.f;
   bool subm = false;
+  bool inverse = false;
   uint32_t max_out = 150000;
   std::string rulebook;
   int precision = SCN_PRECISION_FP16, out_precision = SCN_PRECISION_FP16;
@@ -120,7 +121,7 @@ struct RtTensor {
   bool materialised = false;  // false: fused away, never written
 };
 
-enum class StepKind { InputCount, HashBuild, RulebookSubm, RulebookSparse, Convert, Conv, Add, Relu, Dense, Permute };
+enum class StepKind { InputCount, HashBuild, RulebookSubm, RulebookSparse, RulebookInverse, Convert, Conv, Add, Relu, Dense, Permute };
 
 struct Step {
   StepKind kind;
@@ -161,6 +162,7 @@ struct RbSlot {
   int coord_in = -1, coord_out = -1;
   int ks[3], stride[3], pad[3], dil[3];
   uint32_t max_out = 0;
+  int inverse_of = -1;   // >= 0: the strided rulebook this one swaps (SparseInverseConvolution)
   bool initialised = false;
 };
 
@@ -373,9 +375,46 @@ static bool build_engine(scn_engine& e) {
           return false;
         }
         // rulebook
-        const std::string key = n.rulebook.empty() ? "" : std::string(n.subm ? "subm:" : "conv:") + n.rulebook;
+        const std::string key =
+            n.rulebook.empty() ? "" : std::string(n.inverse ? "inv:" : n.subm ? "subm:" : "conv:") + n.rulebook;
         int rbi = -1;
-        if (!key.empty() && rb_by_key.count(key)) {
+        if (n.inverse) {
+          const auto fw = rb_by_key.find("conv:" + n.rulebook);
+          if (fw == rb_by_key.end() || e.rulebooks[fw->second]->coord_out != x.coord) {
+            set_error("node %s: inverse convolution needs the rulebook '%s' of an earlier strided convolution whose "
+                      "output it runs on", n.name.c_str(), n.rulebook.c_str());
+            return false;
+          }
+          const RbSlot& fs = *e.rulebooks[fw->second];
+          if (memcmp(fs.ks, n.ks, 12) != 0) {
+            set_error("node %s: kernel size differs from that of rulebook '%s'", n.name.c_str(), n.rulebook.c_str());
+            return false;
+          }
+          if (rb_by_key.count(key)) {
+            rbi = rb_by_key[key];
+          } else {
+            auto slot = std::make_unique<RbSlot>();
+            slot->subm = false;
+            slot->inverse_of = fw->second;
+            slot->coord_in = x.coord;
+            slot->coord_out = fs.coord_in;
+            memcpy(slot->ks, fs.ks, 12);
+            memcpy(slot->stride, fs.stride, 12);
+            memcpy(slot->pad, fs.pad, 12);
+            memcpy(slot->dil, fs.dil, 12);
+            rbi = (int)e.rulebooks.size();
+            e.rulebooks.push_back(std::move(slot));
+            rb_by_key[key] = rbi;
+            Step st;
+            st.kind = StepKind::RulebookInverse;
+            st.rulebook = rbi;
+            st.coord = x.coord;
+            st.coord_out = e.rulebooks[rbi]->coord_out;
+            st.node = (int)i;
+            st.label = std::string("rulebook(inverse ") + n.rulebook + ")";
+            e.steps.push_back(st);
+          }
+        } else if (!key.empty() && rb_by_key.count(key)) {
           rbi = rb_by_key[key];
           RbSlot& slot = *e.rulebooks[rbi];
           const bool same = slot.coord_in == x.coord && !memcmp(slot.ks, n.ks, 12) && !memcmp(slot.dil, n.dil, 12) &&
@@ -746,6 +785,15 @@ static int allocate_runtime(scn_engine& e) {
   for (auto& up : e.rulebooks) {
     RbSlot& s = *up;
     const CoordSet& ci = e.coords[s.coord_in];
+    if (s.inverse_of >= 0) {
+      const uint32_t max_in_i = ci.cap, max_out_i = e.coords[s.coord_out].cap;
+      const int kvol_i = s.ks[0] * s.ks[1] * s.ks[2];
+      if (!s.initialised || s.rb.max_in < max_in_i || s.rb.max_out < max_out_i) {
+        if (!s.rb.init(max_in_i, max_out_i, kvol_i)) return SCN_ERR_HIP;
+        s.initialised = true;
+      }
+      continue;
+    }
     if (!s.subm) {
       CoordSet& co = e.coords[s.coord_out];
       uint64_t vol = 1;
@@ -899,6 +947,11 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
       co.lookup = s.rb.out_lookup();
       co.has_lookup = true;
       return SCN_OK;
+    }
+    case StepKind::RulebookInverse: {
+      RbSlot& s = *e.rulebooks[st.rulebook];
+      const RbSlot& f = *e.rulebooks[s.inverse_of];
+      return s.rb.build_inverse(f.rb, e.coords[s.coord_out].n_dev, stream);
     }
     case StepKind::Convert: {
       const RtTensor& x = e.tensors[st.t_in];
@@ -1183,8 +1236,9 @@ int scn_builder_push_sparse_conv(scn_builder* b, const char* name, int x, const 
     set_error("push_sparse_conv(%s): invalid arguments", name ? name : "");
     return -1;
   }
-  if (inverse) {
-    set_error("push_sparse_conv(%s): SparseInverseConvolution is not supported", name ? name : "");
+  if (inverse && (submanifold || !rulebook || !*rulebook)) {
+    set_error("push_sparse_conv(%s): an inverse convolution names the rulebook of an earlier strided convolution",
+              name ? name : "");
     return -1;
   }
   NodeDesc n;
@@ -1225,6 +1279,7 @@ int scn_builder_push_sparse_conv(scn_builder* b, const char* name, int x, const 
   }
   n.in_range = input_dynamic_range;
   n.subm = submanifold != 0;
+  n.inverse = inverse != 0;
   n.max_out = max_output_points ? max_output_points : 150000;
   n.rulebook = rulebook ? rulebook : "";
   n.precision = precision;
@@ -1572,7 +1627,8 @@ int scn_engine_forward(scn_engine* e, void* stream_) {
       SCN_HIP(hipEventRecord(st.ev0, stream));
     }
     const bool coord_step =
-        st.kind == StepKind::HashBuild || st.kind == StepKind::RulebookSubm || st.kind == StepKind::RulebookSparse;
+        st.kind == StepKind::HashBuild || st.kind == StepKind::RulebookSubm || st.kind == StepKind::RulebookSparse ||
+        st.kind == StepKind::RulebookInverse;
     hipStream_t run_on = stream;
     if (dual && coord_step) {
       run_on = e->aux;
@@ -1614,7 +1670,8 @@ int scn_engine_forward(scn_engine* e, void* stream_) {
       SCN_HIP(hipEventRecord(e->ev_fork, stream));
       SCN_HIP(hipStreamWaitEvent(e->aux, e->ev_fork, 0));
     }
-    if (dual && (st.kind == StepKind::RulebookSubm || st.kind == StepKind::RulebookSparse)) {
+    if (dual && (st.kind == StepKind::RulebookSubm || st.kind == StepKind::RulebookSparse ||
+                 st.kind == StepKind::RulebookInverse)) {
       SCN_HIP(hipEventRecord(e->rb_ready[st.rulebook], e->aux));
       e->rb_seq[st.rulebook] = ++aux_seq;
       if (st.kind == StepKind::RulebookSparse) e->coord_rb[e->rulebooks[st.rulebook]->coord_out] = st.rulebook;
@@ -1678,7 +1735,7 @@ int scn_engine_set_profiling(scn_engine* e, int enabled) {
 int scn_engine_num_nodes(const scn_engine* e) { return e ? (int)e->steps.size() : 0; }
 int scn_engine_node_info(scn_engine* e, int node, const char** name, const char** kind, float* last_ms) {
   SCN_REQUIRE(e && node >= 0 && node < (int)e->steps.size(), SCN_ERR_INVALID, "node_info: invalid index");
-  static const char* kinds[] = {"input", "hash", "rulebook_subm", "rulebook_sparse", "convert", "conv", "add", "relu", "dense", "transpose"};
+  static const char* kinds[] = {"input", "hash", "rulebook_subm", "rulebook_sparse", "rulebook_inverse", "convert", "conv", "add", "relu", "dense", "transpose"};
   const Step& s = e->steps[node];
   if (name) *name = s.label.c_str();
   if (kind) *kind = kinds[(int)s.kind];

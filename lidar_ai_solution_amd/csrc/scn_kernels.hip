@@ -742,6 +742,62 @@ int Rulebook::build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev
   return SCN_OK;
 }
 
+// ---- inverse rulebook ---------------------------------------------------------------------------
+// SparseInverseConvolution runs on the rulebook of an earlier strided convolution with the roles
+// swapped: its outputs are that convolution's inputs.  For a fixed kernel offset an input row has at
+// most one output row (o = (i + pad - k dil) / stride), so the swapped rulebook is again a neighbour
+// table: inv[k][i] = o where fwd[k][o] = i.  grid.y = kernel offset.
+__global__ __launch_bounds__(256) void k_invert_nbr(const int32_t* __restrict__ fwd, uint32_t fwd_ld,
+                                                    const uint32_t* n_fwd_out_dev, uint32_t n_fwd_out_bound,
+                                                    int32_t* inv, uint32_t inv_ld, const uint32_t* n_in_dev,
+                                                    uint32_t n_in_bound, uint32_t* n_publish, uint32_t* n_host) {
+  const uint32_t n_out = eff_n(n_fwd_out_dev, n_fwd_out_bound);
+  const uint32_t n_in = eff_n(n_in_dev, n_in_bound);
+  const uint32_t o = blockIdx.x * 256 + threadIdx.x;
+  if (o == 0 && blockIdx.y == 0) {
+    n_publish[0] = n_in;
+    n_publish[1] = n_in;
+    if (n_host) *n_host = n_in;
+  }
+  if (o >= n_out) return;
+  const int32_t i = fwd[(size_t)blockIdx.y * fwd_ld + o];
+  if (i >= 0 && (uint32_t)i < n_in) inv[(size_t)blockIdx.y * inv_ld + (uint32_t)i] = (int32_t)o;
+}
+
+__global__ __launch_bounds__(256) void k_fill_table_rows(int32_t* table, uint32_t ld, uint32_t n, int32_t value) {
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) table[(size_t)blockIdx.y * ld + i] = value;
+}
+
+int Rulebook::build_inverse(const Rulebook& fwd, const uint32_t* n_in_dev, hipStream_t stream) {
+  SCN_REQUIRE(fwd.built && !fwd.subm, SCN_ERR_INVALID, "inverse rulebook: needs a built strided rulebook");
+  SCN_REQUIRE(fwd.geom.kvol <= kvol_cap, SCN_ERR_CAPACITY, "inverse rulebook: kernel volume %d exceeds %d",
+              fwd.geom.kvol, kvol_cap);
+  SCN_REQUIRE(fwd.n_bound_in <= max_out && fwd.n_bound_in <= ld && fwd.n_bound_out <= max_in, SCN_ERR_CAPACITY,
+              "inverse rulebook: %u x %u rows exceed capacity %u x %u", fwd.n_bound_out, fwd.n_bound_in, max_in, max_out);
+  subm = false;
+  geom = fwd.geom;
+  for (int a = 0; a < 3; ++a) {
+    geom.grid_in[a] = fwd.geom.grid_out[a];
+    geom.grid_out[a] = fwd.geom.grid_in[a];
+  }
+  in_indices = fwd.out_indices;
+  out_indices = fwd.in_indices;
+  n_bound_in = fwd.n_bound_out;
+  n_bound_out = fwd.n_bound_in;
+  // every offset's row of the table, up to the row bound, starts as "no neighbour"
+  if (n_bound_out)
+    hipLaunchKernelGGL(k_fill_table_rows, dim3(ceil_div(n_bound_out, 256), geom.kvol), dim3(256), 0, stream,
+                       nbr.as<int32_t>(), ld, n_bound_out, -1);
+  const uint32_t blocks = n_bound_in ? ceil_div(n_bound_in, 256) : 1;  // one block even when empty: it publishes the count
+  hipLaunchKernelGGL(k_invert_nbr, dim3(blocks, geom.kvol), dim3(256), 0, stream, fwd.nbr.as<int32_t>(), fwd.ld,
+                     fwd.n_out_dev(), fwd.n_bound_out, nbr.as<int32_t>(), ld, n_in_dev, n_bound_out,
+                     counters.as<uint32_t>(), host_count.as<uint32_t>());
+  SCN_HIP(hipGetLastError());
+  built = true;
+  return SCN_OK;
+}
+
 // ---- pair compaction: nbr[k][o] -> (in,out) lists per offset, ordered by (k, out) -------------
 __global__ __launch_bounds__(256) void k_pair_count(const int32_t* __restrict__ nbr, uint32_t ld,
                                                     const uint32_t* n_out_dev, uint32_t n_bound, uint32_t* counts) {
@@ -2267,6 +2323,10 @@ int scn_rulebook_build_sparse(scn_rulebook* rb, const int32_t* indices_dev, uint
               "null pointer");
   return rb->rb.build_sparse(indices_dev, n, n_dev, grid, ksize, stride, padding, dilation, nullptr,
                              (hipStream_t)stream);
+}
+int scn_rulebook_build_inverse(scn_rulebook* rb, const scn_rulebook* forward, const uint32_t* n_in_dev, void* stream) {
+  SCN_REQUIRE(rb && forward, SCN_ERR_INVALID, "null pointer");
+  return rb->rb.build_inverse(forward->rb, n_in_dev, (hipStream_t)stream);
 }
 const int32_t* scn_rulebook_nbr(const scn_rulebook* rb) { return rb ? rb->rb.nbr.as<int32_t>() : nullptr; }
 uint32_t scn_rulebook_nbr_ld(const scn_rulebook* rb) { return rb ? rb->rb.ld : 0; }

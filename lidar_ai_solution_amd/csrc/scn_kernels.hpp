@@ -74,6 +74,9 @@ struct Rulebook {
   int build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3], const int ks[3],
                    const int stride[3], const int pad[3], const int dil[3], const CoordLookup* shared_lookup,
                    hipStream_t stream);
+  // the rulebook of SparseInverseConvolution: fwd (strided, built) with inputs and outputs swapped; n_in_dev
+  // (nullable) is the device-side row count of fwd's input, which becomes this rulebook's output count
+  int build_inverse(const Rulebook& fwd, const uint32_t* n_in_dev, hipStream_t stream);
   CoordLookup out_lookup() const;  // strided: rows of the output tensor from bitmap ranks
   int pairs(int32_t* pair_in, int32_t* pair_out, int64_t* offsets, uint64_t capacity, hipStream_t stream);
   const uint32_t* n_out_dev() const { return counters.as<uint32_t>(); }

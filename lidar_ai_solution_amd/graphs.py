@@ -34,7 +34,7 @@ class _Builder:
         return t
 
     def conv(self, x: str, cin: int, cout: int, ksize, stride=(1, 1, 1), padding=(0, 0, 0), subm=False,
-             rulebook="", activation="ReLU", tag="") -> str:
+             rulebook="", activation="ReLU", tag="", inverse=False) -> str:
         i = self.nconv
         self.nconv += 1
         w = (self.rng.standard_normal((cout, *ksize, cin)) * self.std).astype(np.float16)
@@ -45,7 +45,7 @@ class _Builder:
         self.nodes.append(Node("SparseConvolution", f"conv{i}", [x, f"spconv{i}.weight", f"spconv{i}.bias"], [y], {
             "ndim": 3, "in_channels": cin, "out_channels": cout,
             "kernel_size": list(ksize), "stride": list(stride), "padding": list(padding), "dilation": [1, 1, 1],
-            "output_bound": 200000, "transposed": 0, "inverse": 0, "groups": 1,
+            "output_bound": 200000, "transposed": 0, "inverse": int(inverse), "groups": 1,
             "subm": int(subm), "rulebook": rulebook, "activation": activation, "tag": tag,
         }))
         return y
@@ -151,6 +151,30 @@ def single_subm_layer(seed: int = 0, cin: int = 16, cout: int = 16) -> Graph:
     return Graph(["0"], [y], b.nodes, b.inits)
 
 
+def unet_scn(seed: int = 0, in_channels: int = 5, channels: Sequence[int] = (16, 32, 64), weight_std: float = 0.05
+             ) -> Tuple[Graph, Dict[str, str]]:
+    """Small encoder-decoder (two strided convolutions down, two SparseInverseConvolution nodes back up
+    on the same rulebooks, skip connections by Add): the shape of spconv's segmentation networks, with a
+    sparse graph output.  Exercises the `inverse` attribute of the dialect."""
+    b = _Builder(seed, weight_std)
+    c0, c1, c2 = channels
+    x0 = b.conv("0", in_channels, c0, (3, 3, 3), subm=True, rulebook="s0", tag="enc0.in")
+    x0 = b.block(x0, c0, "s0", "enc0.res")
+    x1 = b.conv(x0, c0, c1, (3, 3, 3), (2, 2, 2), (1, 1, 1), rulebook="down1", tag="enc1.down")
+    x1 = b.block(x1, c1, "s1", "enc1.res")
+    x2 = b.conv(x1, c1, c2, (3, 3, 3), (2, 2, 2), (1, 1, 1), rulebook="down2", tag="enc2.down")
+    x2 = b.block(x2, c2, "s2", "enc2.res")
+    u1 = b.conv(x2, c2, c1, (3, 3, 3), (2, 2, 2), (1, 1, 1), rulebook="down2", activation="None", tag="dec1.up",
+                inverse=True)
+    u1 = b.relu(b.add(u1, x1, tag="dec1.skip"))
+    u1 = b.block(u1, c1, "s1", "dec1.res")
+    u0 = b.conv(u1, c1, c0, (3, 3, 3), (2, 2, 2), (1, 1, 1), rulebook="down1", activation="None", tag="dec0.up",
+                inverse=True)
+    u0 = b.relu(b.add(u0, x0, tag="dec0.skip"))
+    tags = _strip_tags(b.nodes)
+    return Graph(["0"], [u0], b.nodes, b.inits), tags
+
+
 # --------------------------------------------------------------------------- int8 plans
 def weight_dynamic_ranges(w: np.ndarray) -> List[float]:
     """Per-output-channel amax of `[Cout, K0, K1, K2, Cin]` fp16 weights (quantizer axis 0)."""
@@ -163,7 +187,7 @@ def apply_int8_plan(graph: Graph, tags: Dict[str, str], tensor_amax: Dict[str, f
     tensor_amax maps a tensor name to the calibrated per-tensor amax of its values.  Conv nodes get
     `input_dynamic_range` = amax of their input; Add nodes get one shared range for both inputs
     (`exptool.py:226-227`): the larger of the two input amaxes.
-    plan: "centerpoint" or "bevfusion".
+    plan: "centerpoint", "bevfusion" or "all-int8" (every convolution and Add computes and stores int8).
     """
     fp16_compute: set = set()
     fp16_output: set = set()
@@ -173,6 +197,8 @@ def apply_int8_plan(graph: Graph, tags: Dict[str, str], tensor_amax: Dict[str, f
     elif plan == "bevfusion":
         fp16_compute = {"conv_input"}
         fp16_output = {"conv_out"}
+    elif plan == "all-int8":
+        pass
     else:
         raise ValueError(plan)
     for n in graph.nodes:

@@ -20,6 +20,9 @@ Precision rules stated by this build (the closed engine's are not recoverable):
   * int8 conv: Wq from the per-channel weight ranges the same way, acc int32,
     y = acc * (s_x * s_w[c]) + bias (two fp32 roundings), ReLU, then int8 or fp16 store.
   * Add: value of an int8 operand is q * (amax(tensor)/127); one fp32 add; same stores.
+  * SparseInverseConvolution (parity unpinned: no reference vector exists): the transposed convolution
+    on the named strided rulebook, out[i] += W[k] x[o] for each of its pairs (i, o, k), kernel not
+    flipped; pinned against torch's conv_transpose3d under that rule.
 """
 from __future__ import annotations
 
@@ -152,6 +155,24 @@ def rulebook_sparse(indices: np.ndarray, grid, ksize, stride, padding, dilation=
     assert npairs >= 0
     return Rulebook(pin[:npairs].copy(), pout[:npairs].copy(), offs, oidx[:n_out.value].copy(),
                     [int(v) for v in ogrid], n_out.value, n_tot.value)
+
+
+def rulebook_inverse(rb: Rulebook, in_indices: np.ndarray, in_grid) -> Rulebook:
+    """Rulebook of a SparseInverseConvolution on the rulebook `rb` of a strided convolution whose input
+    was (in_indices, in_grid): the same pairs with input and output swapped, so the outputs are that
+    convolution's input rows; the kernel offset of a pair (and with it the weight slice) stays.
+    (`inverse` argument of push_sparse_conv, libraries/3DSparseConvolution/libspconv/include/spconv/engine.hpp:139-156;
+    the arithmetic behind it is not in the reference's sources: this rule is the transposed
+    convolution, out[i] += W[k] x[o] for every pair (i, o, k) of the forward rulebook.)"""
+    pin = np.empty_like(rb.pair_in)
+    pout = np.empty_like(rb.pair_out)
+    for k in range(len(rb.offsets) - 1):
+        a, b = int(rb.offsets[k]), int(rb.offsets[k + 1])
+        order = np.lexsort((rb.pair_out[a:b], rb.pair_in[a:b]))   # by new output (old input), then new input
+        pin[a:b] = rb.pair_out[a:b][order]
+        pout[a:b] = rb.pair_in[a:b][order]
+    idx = np.ascontiguousarray(in_indices, np.int32)
+    return Rulebook(pin, pout, rb.offsets.copy(), idx, list(in_grid), idx.shape[0])
 
 
 # ------------------------------------------------------------------------------- conv + elementwise
@@ -361,7 +382,15 @@ def run_graph(graph, features_f16: np.ndarray, indices: np.ndarray, grid, precis
             bias = graph.initializers[n.inputs[2]].astype(np.float32)
             ks, dil = a["kernel_size"], a.get("dilation", [1, 1, 1]) or [1, 1, 1]
             key = a.get("rulebook", "")
-            if a.get("subm", 0):
+            if a.get("inverse", 0):
+                fwd = rb_cache.get("conv:" + key)
+                if fwd is None or not np.array_equal(fwd.out_indices, x.indices):
+                    raise ValueError(f"node {n.name}: inverse convolution needs the rulebook '{key}' of an earlier "
+                                     f"strided convolution whose output it runs on")
+                rb = rb_cache.get("inv:" + key)
+                if rb is None:
+                    rb = rb_cache["inv:" + key] = rulebook_inverse(fwd, fwd.in_indices, fwd.in_grid)
+            elif a.get("subm", 0):
                 ck = "subm:" + key
                 rb = rb_cache.get(ck) if key else None
                 if rb is None:
@@ -374,6 +403,7 @@ def run_graph(graph, features_f16: np.ndarray, indices: np.ndarray, grid, precis
                 if rb is None:
                     rb = rulebook_sparse(x.indices, x.grid, ks, a["stride"], a["padding"], dil,
                                          int(a.get("output_bound", 150000)))
+                    rb.in_indices, rb.in_grid = x.indices, list(x.grid)
                     if key:
                         rb_cache[ck] = rb
             relu = a.get("activation", "") == "ReLU"

@@ -75,6 +75,11 @@ class GpuRulebook:
                                                    i3(pad), i3(dil), stream()))
         self.kvol = int(np.prod(ksize))
 
+    def build_inverse(self, forward, n_in_dev=None):
+        self._fwd = forward
+        capi.check(self.L.scn_rulebook_build_inverse(self.h, forward.h, ptr(n_in_dev), stream()))
+        self.kvol = forward.kvol
+
     def n_out(self):
         return read_u32(self.L.scn_rulebook_num_out_dev(self.h))
 

@@ -233,6 +233,49 @@ def test_bevfusion_int8_graph_xyz(bevfusion_input):
     assert np.array_equal(got.view(np.uint16), rec[g8.nodes[-1].name]["out"].view(np.uint16))
 
 
+def test_unet_with_inverse_convolutions(centerpoint_input, tmp_path):
+    """Encoder-decoder with two SparseInverseConvolution nodes on the rulebooks of its strided convolutions,
+    skip connections and a sparse graph output: fp16 within the stated tolerance, the all-int8 plan bit-exact
+    in every accumulator and every stored tensor; one and two streams, and through an ONNX file."""
+    feats, idx = centerpoint_input
+    n = 30000
+    feats, idx = feats[:n], idx[:n]
+    g16, tags = graphs.unet_scn(seed=3)
+    note("fp16 U-Net-shaped graph (inverse convolutions) on 30,000 fixture voxels, from an ONNX file")
+    path = str(tmp_path / "unet.scn.onnx")
+    onnx_dialect.save(g16, path)
+    eng = Engine.from_onnx(path, "fp16")
+    _run_engine(eng, feats, idx, GRID_ZYX)
+    out = eng.output(0)
+    assert not out.dense
+    got_f, got_i = out.torch()
+    ref = O.run_graph(g16, feats, idx, GRID_ZYX, "fp16")[g16.outputs[0]]
+    assert np.array_equal(got_i.cpu().numpy()[:n], idx) and np.array_equal(ref.indices, idx)
+    got = got_f.cpu().numpy()[:n, :ref.feat.shape[1]]
+    maxabs, cos, refmax = _compare_dense(got, ref.feat)
+    print(f"fp16 unet: max-abs {maxabs:.3e} (ref max {refmax:.3e}), cosine {cos:.6f}")
+    assert maxabs <= FP16_REL * refmax and cos >= FP16_COS
+    note("all-int8 plan, every tensor kept: accumulators and stored tensors bit-exact")
+    amax = _oracle_calibration(g16, feats, idx, GRID_ZYX)
+    g8, tags8 = graphs.unet_scn(seed=3)
+    graphs.apply_int8_plan(g8, tags8, amax, "all-int8")
+    rec = {}
+    ref8 = O.run_graph(g8, feats, idx, GRID_ZYX, "int8", rec)[g8.outputs[0]]
+    eng8 = Engine.from_graph(g8, "int8", keep_all=True)
+    _run_engine(eng8, feats, idx, GRID_ZYX)
+    nacc, nout = _check_every_layer(g8, eng8, rec)
+    print(f"bit-exact: {nacc} int32 accumulator tensors, {nout} int8 tensors")
+    assert nacc == 13 and nout >= 13
+    note("fused engine, auxiliary stream, two forwards with different row counts")
+    eng_f = Engine.from_graph(g8, "int8", with_auxiliary_stream=True)
+    for m in (n, n - 4321, n):
+        r = O.run_graph(g8, feats[:m], idx[:m], GRID_ZYX, "int8")[g8.outputs[0]]
+        _run_engine(eng_f, feats[:m], idx[:m], GRID_ZYX)
+        gf, _ = eng_f.output(0).torch()
+        assert np.array_equal(gf.cpu().numpy()[:m, :r.feat.shape[1]], r.feat), m
+    assert np.count_nonzero(ref8.feat) > 10000   # (the last tensor has no consumer that fixes a range: stored fp16)
+
+
 def test_engine_edge_cases(cp_models, centerpoint_input):
     feats, idx = centerpoint_input
     g16, g8 = cp_models

@@ -414,6 +414,53 @@ def test_convert_add_and_dense():
     assert np.array_equal(out.cpu().numpy().view(np.uint16), O.scatter_dense(O.dequantize(qf, 6.35), idx, dims).view(np.uint16))
 
 
+@pytest.mark.parametrize("cin,cout", [(32, 16), (128, 64)])
+def test_inverse_rulebook_and_int8_conv(cin, cout, centerpoint_input):
+    """SparseInverseConvolution: the swapped rulebook of a strided convolution (pairs identical to the
+    oracle's, output rows = the forward convolution's input rows, also with a device-side input count)
+    and an int8 convolution through it, bit-exact."""
+    _, idx_all = centerpoint_input
+    rng = np.random.default_rng(cin)
+    n = 20000
+    idx = idx_all[:n]
+    grid = (41, 1440, 1440)
+    ks, st, pad = (3, 3, 3), (2, 2, 2), (1, 1, 1)
+    note(f"inverse rulebook of a stride-2 3x3x3 convolution on {n} fixture voxels, int8 conv {cin}->{cout}")
+    ref_f = O.rulebook_sparse(idx, grid, ks, st, pad, max_out=n * 2)
+    ref_i = O.rulebook_inverse(ref_f, idx, grid)
+    d_idx = to_dev(idx)
+    fwd = GpuRulebook(n, n * 2, 27)
+    fwd.build_sparse(d_idx, n, grid, ks, st, pad)
+    m = fwd.n_out()
+    assert m == ref_f.n_out
+    inv = GpuRulebook(n * 2, n, 27)
+    inv.build_inverse(fwd)
+    assert inv.n_out() == n
+    pin, pout, offs = inv.pairs(ref_i.num_pairs + 16)
+    assert np.array_equal(offs, ref_i.offsets) and np.array_equal(pin, ref_i.pair_in) and np.array_equal(pout, ref_i.pair_out)
+    assert np.array_equal(inv.out_indices(), idx)
+    x = rng.integers(-127, 128, (m, cin)).astype(np.int8)
+    w, b, ranges = _weights(rng, cout, ks, cin)
+    x_range, out_range = 4.2, 7.7
+    wq, s_w = O.quantize_weights(w, ranges)
+    acc_ref = O.conv_int8_acc(x, wq, ref_i)
+    scale = (np.float32(x_range) / np.float32(127) * s_w).astype(np.float32)
+    conv = GpuConv(w, ranges, b, capi.PRECISION_INT8)
+    out, acc = conv.forward(inv, to_dev(x), n, x_range=x_range, relu=True, out_int8=True, out_range=out_range, want_acc=True)
+    assert np.array_equal(acc.cpu().numpy(), acc_ref)
+    assert np.array_equal(out.cpu().numpy(), O.epilogue(acc_ref, scale, b.astype(np.float32), True, True, out_range))
+    note("device-side input count below the bound: rows past it neither appear as outputs nor as neighbours")
+    k = n - 777
+    cnt = to_dev(np.array([k], np.uint32))
+    ref_f2 = O.rulebook_sparse(idx[:k], grid, ks, st, pad, max_out=n * 2)
+    ref_i2 = O.rulebook_inverse(ref_f2, idx[:k], grid)
+    fwd.build_sparse(d_idx, n, grid, ks, st, pad, n_dev=cnt)
+    inv.build_inverse(fwd, n_in_dev=cnt)
+    assert inv.n_out() == k
+    pin, pout, offs = inv.pairs(ref_i2.num_pairs + 16)
+    assert np.array_equal(offs, ref_i2.offsets) and np.array_equal(pin, ref_i2.pair_in) and np.array_equal(pout, ref_i2.pair_out)
+
+
 def test_scatter_dense_with_row_map():
     """The dense-major variant (row map, no clear, whole 16-byte stores) against the oracle: fp16 and int8
     rows, channel counts that are not a multiple of 8, permuted spatial axes, a device-side row count, a

@@ -242,6 +242,40 @@ def test_rulebook_and_int8_conv_against_dense_conv3d(case):
     assert np.allclose(accf, gotf, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("case", [c for c in CONV_CASES if not c[6]])
+def test_inverse_rulebook_against_dense_conv_transpose3d(case):
+    """SparseInverseConvolution on a strided rulebook == torch conv_transpose3d (float64, exact for int8
+    data) of the zero-filled dense output grid, sampled at the forward convolution's input sites.  A kernel
+    flip, a swapped operand or a wrong offset fails this."""
+    grid, n, ks, st, pad, dil, _ = case
+    rng = np.random.default_rng(hash(case) % (2 ** 31) + 1)
+    cin, cout = 6, 4          # of the inverse convolution: cin = channels on the coarse grid
+    idx = _random_sparse(rng, grid, n)
+    fwd = O.rulebook_sparse(idx, grid, ks, st, pad, dil)
+    inv = O.rulebook_inverse(fwd, idx, grid)
+    assert inv.n_out == n and np.array_equal(inv.out_indices, idx) and inv.out_grid == list(grid)
+    assert inv.num_pairs == fwd.num_pairs and np.array_equal(inv.offsets, fwd.offsets)
+    for k in range(len(fwd.offsets) - 1):     # same pairs per offset, roles swapped, ordered by output
+        a, b = int(fwd.offsets[k]), int(fwd.offsets[k + 1])
+        assert sorted(zip(inv.pair_out[a:b], inv.pair_in[a:b])) == sorted(zip(fwd.pair_in[a:b], fwd.pair_out[a:b]))
+        assert np.all(np.diff(inv.pair_out[a:b]) > 0)      # an input row has one output row per offset
+    m = fwd.n_out
+    x = rng.integers(-127, 128, (m, cin)).astype(np.int8)
+    wq = rng.integers(-127, 128, (int(np.prod(ks)), cout, cin)).astype(np.int8)
+    acc = O.conv_int8_acc(x, wq, inv)
+    og = fwd.out_grid
+    oi = fwd.out_indices
+    dense = torch.zeros(1, cin, *og, dtype=torch.float64)
+    dense[0, :, oi[:, 1], oi[:, 2], oi[:, 3]] = torch.from_numpy(x.astype(np.float64)).T
+    w = torch.from_numpy(wq.astype(np.float64)).reshape(*ks, cout, cin).permute(4, 3, 0, 1, 2).contiguous()  # [Cin, Cout, k]
+    opad = [grid[a] - ((og[a] - 1) * st[a] - 2 * pad[a] + dil[a] * (ks[a] - 1) + 1) for a in range(3)]
+    assert all(0 <= opad[a] < max(st[a], dil[a]) or opad[a] == 0 for a in range(3))
+    y = torch.nn.functional.conv_transpose3d(dense, w, stride=st, padding=pad, output_padding=opad, dilation=dil)[0]
+    assert list(y.shape[1:]) == list(grid)
+    got = y[:, idx[:, 1], idx[:, 2], idx[:, 3]].T.numpy()
+    assert np.array_equal(acc.astype(np.float64), got)
+
+
 def test_sparse_rulebook_truncation_keeps_lowest_outputs():
     rng = np.random.default_rng(5)
     grid = (7, 12, 10)
