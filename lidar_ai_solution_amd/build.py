@@ -26,17 +26,36 @@ def sources():
     return src
 
 
-def build(verbose: bool = False) -> str:
-    os.makedirs(LIB_DIR, exist_ok=True)
-    cmd = ["hipcc", *FLAGS, "-I" + os.path.join(ROOT, "include"), *sources(), "-o", LIB_PATH]
+def _run(cmd, verbose):
     if verbose:
-        print(" ".join(cmd))
+        print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
     if proc.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
+        raise RuntimeError("hipcc failed: " + " ".join(cmd) + "\n" + out)
     if verbose and out.strip():
         print(out)
+
+
+def build(verbose: bool = False, jobs: int = 0) -> str:
+    """Compiles every source to an object file (side by side, `jobs` at a time) and links the library."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    os.makedirs(LIB_DIR, exist_ok=True)
+    obj_dir = os.path.join(LIB_DIR, "obj")
+    os.makedirs(obj_dir, exist_ok=True)
+    compile_flags = [f for f in FLAGS if f not in ("-shared", "-no-hip-rt")]
+    jobs_ = jobs or min(8, os.cpu_count() or 1)
+    objs = []
+    cmds = []
+    for src in sources():
+        obj = os.path.join(obj_dir, os.path.basename(src) + ".o")
+        objs.append(obj)
+        cmds.append(["hipcc", *compile_flags, "-I" + os.path.join(ROOT, "include"), "-c", src, "-o", obj])
+    with ThreadPoolExecutor(max_workers=jobs_) as pool:
+        list(pool.map(lambda c: _run(c, verbose), cmds))
+    _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-fvisibility=hidden", "-no-hip-rt", *objs, "-o", LIB_PATH],
+         verbose)
     return LIB_PATH
 
 

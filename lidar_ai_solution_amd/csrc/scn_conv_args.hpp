@@ -1,0 +1,46 @@
+// Arguments of the convolution kernels and the per-element-type launchers.
+#pragma once
+
+#include "scn_kernels.hpp"
+
+namespace scn {
+
+struct ConvArgs {
+  const char* x;
+  uint32_t x_ld_bytes;
+  const int32_t* nbr;
+  uint32_t nbr_ld;
+  int kvol;
+  const uint32_t* n_out_dev;
+  uint32_t n_bound;
+  const uint4* wfrag;
+  int steps;
+  const float* wscale;
+  const float* bias;
+  int cout;
+  float x_scale;            // amax_x / 127
+  int relu;
+  int out_dtype;
+  float out_r;              // 127 / amax_out
+  char* out;
+  uint32_t out_ld;
+  void* acc;
+  const char* res;
+  int res_dtype;
+  float res_scale;          // amax_res / 127
+  uint32_t res_ld;
+  int mid_dtype;
+  float mid_s, mid_r;       // amax_mid / 127, 127 / amax_mid
+  float a_rq_s, a_rq_r;     // re-quantisation of an fp16 operand by an int8 Add (0 = none)
+  float b_rq_s, b_rq_r;
+  int relu2;
+  int out_vec16;     // output rows are 16-byte aligned and a multiple of 16 bytes: 16-byte stores allowed
+  const char* zrow;  // 512 bytes of zeros (gather source of lanes without a neighbour), then 64 words of -1
+};
+
+// Launch the kernel for these weights (one definition per element type, each in its own translation unit).
+// n_hint: expected number of output rows.  Returns false when no kernel covers the shape.
+bool conv_dispatch_int8(const ConvWeights& w, uint32_t n_hint, ConvArgs& a, hipStream_t stream);
+bool conv_dispatch_fp16(const ConvWeights& w, uint32_t n_hint, ConvArgs& a, hipStream_t stream);
+
+}  // namespace scn

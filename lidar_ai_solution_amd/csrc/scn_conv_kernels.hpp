@@ -1,0 +1,660 @@
+// Convolution kernels of the SCN path (gfx950) and their launch dispatch, as templates over the element
+// type: included by one translation unit per element type so that the two sets of instantiations
+// compile side by side.
+#pragma once
+
+#include "scn_conv_args.hpp"
+#include "scn_device.hpp"
+
+#include <cstdlib>
+#include <cstring>
+
+namespace scn {
+
+// --------------------------------------------------------------------------------------------
+// gather-GEMM convolution
+// --------------------------------------------------------------------------------------------
+// Operand mapping of v_mfma_i32_16x16x64_i8 / v_mfma_f32_16x16x32_f16 (D = A x B + C, wave64):
+//   A (16 x K): lane l supplies row  m = l % 16, the 16 bytes of K-block l / 16
+//   B (K x 16): lane l supplies col  n = l % 16, the 16 bytes of K-block l / 16
+//   D (16 x 16): lane l holds col n = l % 16, rows m = 4 * (l / 16) + {0,1,2,3}
+// Rows of A are output channels (weights, pre-packed on the host in exactly this order), columns of
+// B are voxels: the 16 bytes a lane needs are 16 contiguous input channels of one gathered row, so
+// a gathered row goes from memory straight into the MFMA operand with one 16-byte load, and each
+// lane ends up with 4 consecutive output channels of one voxel, stored with one 4/8-byte store.
+// One 16-byte "chunk" = 16 int8 or 8 fp16 input channels; K-step s consumes chunks 4s..4s+3 of the
+// sequence (offset 0 chunk 0, offset 0 chunk 1, ..., offset kvol-1 chunk CHUNKS-1).
+
+
+template <int EL>
+struct Mma;
+template <>
+struct Mma<0> {
+  using Acc = v4i;
+  static __device__ __forceinline__ Acc run(const v4i a, const v4i b, Acc c) {
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ Acc run(const uint4& a, const uint4& b, Acc c) {
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(v4i, a), __builtin_bit_cast(v4i, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<1> {
+  using Acc = v4f;
+  static __device__ __forceinline__ Acc run(const v4i a, const v4i b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ Acc run(const uint4& a, const uint4& b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+};
+
+// Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2.  Giving XCD x the
+// x-th contiguous eighth of the row tiles keeps the rows a tile gathers (spatial neighbours, i.e.
+// nearby rows in canonical order) inside one L2 instead of spreading every row over all eight.
+// Returns false when this workgroup has no tile.
+__device__ __forceinline__ bool xcd_tile(uint32_t n, uint32_t rows_per_block, uint32_t* tile) {
+  const uint32_t tiles = (n + rows_per_block - 1) / rows_per_block;
+  const uint32_t per = (tiles + 7) >> 3;
+  const uint32_t xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+  *tile = xcd * per + j;
+  return j < per && *tile < tiles;
+}
+
+// Fused epilogue of 4 consecutive channels of one row: bias, requantisation scale, ReLU, residual add
+// (with the mid-quantisation the un-fused graph would have applied), second ReLU.  Also dumps the raw
+// accumulators when asked to.  y[] receives the values to store.
+template <int EL>
+__device__ __forceinline__ void epilogue_values(const ConvArgs& a, uint32_t row, int co,
+                                                const typename Mma<EL>::Acc& acc, float y[4]) {
+  const float4 bs = *reinterpret_cast<const float4*>(a.bias + co);
+  const float b4[4] = {bs.x, bs.y, bs.z, bs.w};
+  if (EL == 0) {
+    const float4 ws = *reinterpret_cast<const float4*>(a.wscale + co);
+    const float w4[4] = {ws.x, ws.y, ws.z, ws.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float sc = a.x_scale * w4[j];         // s_x * s_w[c], one fp32 rounding
+      const float m = (float)acc[j] * sc;          // fp32 multiply
+      y[j] = m + b4[j];                            // fp32 add (the library is built with -ffp-contract=off)
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) y[j] = (float)acc[j] + b4[j];
+  }
+  if (a.acc) {
+    if (EL == 0)
+      *reinterpret_cast<v4i*>((int32_t*)a.acc + (size_t)row * a.cout + co) = __builtin_bit_cast(v4i, acc);
+    else
+      *reinterpret_cast<v4f*>((float*)a.acc + (size_t)row * a.cout + co) = __builtin_bit_cast(v4f, acc);
+  }
+  if (a.relu) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) y[j] = y[j] > 0.f ? y[j] : 0.f;
+  }
+  if (a.res) {
+    // value of the un-fused conv output as its consumer (the Add) would have read it
+    float rv[4];
+    if (a.res_dtype == SCN_DTYPE_INT8) {
+      const char4 r = *reinterpret_cast<const char4*>(a.res + (size_t)row * a.res_ld + co);
+      rv[0] = (float)r.x * a.res_scale;
+      rv[1] = (float)r.y * a.res_scale;
+      rv[2] = (float)r.z * a.res_scale;
+      rv[3] = (float)r.w * a.res_scale;
+    } else {
+      const _Float16* r = reinterpret_cast<const _Float16*>(a.res) + (size_t)row * a.res_ld + co;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        rv[j] = (float)r[j];
+        if (a.b_rq_r > 0.f) rv[j] = quant_f(rv[j], a.b_rq_r) * a.b_rq_s;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float v;
+      if (a.mid_dtype == SCN_DTYPE_INT8) {
+        v = quant_f(y[j], a.mid_r) * a.mid_s;
+      } else {
+        v = half_round(y[j]);
+        if (a.a_rq_r > 0.f) v = quant_f(v, a.a_rq_r) * a.a_rq_s;
+      }
+      v = v + rv[j];
+      if (a.relu2) v = v > 0.f ? v : 0.f;
+      y[j] = v;
+    }
+  }
+}
+
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ char4 pack_int8(const ConvArgs& a, const float y[4]) {
+  char4 q;
+  q.x = (signed char)quant_f(y[0], a.out_r);
+  q.y = (signed char)quant_f(y[1], a.out_r);
+  q.z = (signed char)quant_f(y[2], a.out_r);
+  q.w = (signed char)quant_f(y[3], a.out_r);
+  return q;
+}
+
+__device__ __forceinline__ v4h pack_fp16(const float y[4]) {
+  return v4h{(_Float16)y[0], (_Float16)y[1], (_Float16)y[2], (_Float16)y[3]};
+}
+
+// Stores 4 consecutive channels of one row after the fused epilogue.
+template <int EL>
+__device__ __forceinline__ void epilogue_store(const ConvArgs& a, uint32_t row, int co, const typename Mma<EL>::Acc& acc) {
+  float y[4];
+  epilogue_values<EL>(a, row, co, acc, y);
+  if (a.out_dtype == SCN_DTYPE_INT8)
+    *reinterpret_cast<char4*>(a.out + (size_t)row * a.out_ld + co) = pack_int8(a, y);
+  else
+    *reinterpret_cast<v4h*>(reinterpret_cast<_Float16*>(a.out) + (size_t)row * a.out_ld + co) = pack_fp16(y);
+}
+
+// Row-split kernel: each wave owns 16*NT output rows and all MT*16 output channels; both operands
+// come straight from global memory / L2 (weights: coalesced 1 KB fragments; features: gathered rows).
+template <int EL, int CHUNKS, int MT, int NT>
+__global__ __launch_bounds__(256) void k_conv_rows(const ConvArgs a) {
+  using Acc = typename Mma<EL>::Acc;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const uint32_t n = eff_n(a.n_out_dev, a.n_bound);
+  uint32_t tile;
+  if (!xcd_tile(n, 64u * NT, &tile)) return;
+  const uint32_t row0 = (tile * 4 + wave) * (16 * NT);
+  if (row0 >= n) return;
+  Acc acc[MT][NT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int u = 0; u < NT; ++u) acc[t][u] = Acc{0, 0, 0, 0};
+  const uint4* wf = a.wfrag + lane;
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  uint32_t rows[NT];
+#pragma unroll
+  for (int u = 0; u < NT; ++u) rows[u] = row0 + u * 16 + lr;
+
+  if constexpr (CHUNKS >= 4) {
+    constexpr int SPK = CHUNKS / 4;  // K-steps per kernel offset
+    for (int k = 0; k < a.kvol; ++k) {
+      int32_t idx[NT];
+      bool any = false;
+#pragma unroll
+      for (int u = 0; u < NT; ++u) {
+        idx[u] = rows[u] < n ? a.nbr[(size_t)k * a.nbr_ld + rows[u]] : -1;
+        any |= idx[u] >= 0;
+      }
+      if (!__any(any)) continue;  // no row of this wave has a neighbour at this offset
+#pragma unroll
+      for (int ss = 0; ss < SPK; ++ss) {
+        uint4 b[NT];
+#pragma unroll
+        for (int u = 0; u < NT; ++u) {
+          b[u] = *reinterpret_cast<const uint4*>(a.x + (size_t)(idx[u] >= 0 ? idx[u] : 0) * a.x_ld_bytes +
+                                                 (ss * 4 + lg) * 16);
+          if (idx[u] < 0) b[u] = zero;
+        }
+        const int s = k * SPK + ss;
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          const uint4 av = wf[(size_t)(s * MT + t) * 64];
+#pragma unroll
+          for (int u = 0; u < NT; ++u) acc[t][u] = Mma<EL>::run(av, b[u], acc[t][u]);
+        }
+      }
+    }
+  } else {
+    const int total_chunks = a.kvol * CHUNKS;
+    for (int s = 0; s < a.steps; ++s) {
+      const int g = 4 * s + lg;
+      const int k = g / CHUNKS, c = g % CHUNKS;
+      const bool gv = g < total_chunks;
+      uint4 b[NT];
+      bool any = false;
+#pragma unroll
+      for (int u = 0; u < NT; ++u) {
+        int32_t idx = -1;
+        if (gv && rows[u] < n) idx = a.nbr[(size_t)k * a.nbr_ld + rows[u]];
+        any |= idx >= 0;
+        b[u] = *reinterpret_cast<const uint4*>(a.x + (size_t)(idx >= 0 ? idx : 0) * a.x_ld_bytes + c * 16);
+        if (idx < 0) b[u] = zero;
+      }
+      if (!__any(any)) continue;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const uint4 av = wf[(size_t)(s * MT + t) * 64];
+#pragma unroll
+        for (int u = 0; u < NT; ++u) acc[t][u] = Mma<EL>::run(av, b[u], acc[t][u]);
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < NT; ++u) {
+    if (rows[u] >= n) continue;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) epilogue_store<EL>(a, rows[u], t * 16 + lg * 4, acc[t][u]);
+  }
+}
+
+// --------------------------------------------------------------------------------------------
+// 32x32 MFMA variant (output channels >= 32).
+// Measured issue rates on MI355X (independent accumulators, 4 waves per SIMD): v_mfma_i32_32x32x32_i8
+// 4.77 POP/s and v_mfma_f32_32x32x16_f16 2.39 PFLOP/s, against 2.7 POP/s / 1.35 PFLOP/s for the
+// 16x16x64 / 16x16x32 forms: only the 32x32 forms reach the matrix peak, so wide layers use them.
+// Operand mapping (wave64):  A (32 x K): lane l supplies row m = l % 32, the 16 bytes of K-half l / 32
+//                            B (K x 32): lane l supplies col n = l % 32, the 16 bytes of K-half l / 32
+//                            D (32 x 32): lane l holds col n = l % 32, rows 8 * (j / 4) + 4 * (l / 32) + j % 4
+// Rows of A are output channels, columns of B voxels; K-step s consumes chunks 2s and 2s+1 of the
+// (offset, chunk) sequence.
+template <int EL>
+struct Mma32;
+template <>
+struct Mma32<0> {
+  using Acc = v16i;
+  using Acc4 = v4i;
+  static __device__ __forceinline__ Acc run(const v4i a, const v4i b, Acc c) {
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma32<1> {
+  using Acc = v16f;
+  using Acc4 = v4f;
+  static __device__ __forceinline__ Acc run(const v4i a, const v4i b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+};
+
+// --------------------------------------------------------------------------------------------
+// LDS-staged gather kernel (32x32 MFMA, output channels >= 32).
+// What bounds the register-gather kernels above is the vector-memory path, not the matrix cores: a
+// gather in MFMA operand order (32 rows x 2 lanes x 16 B) costs ~97 cycles of a CU's texture pipe per
+// instruction, one whose 8 adjacent lanes read one row's 128 contiguous bytes ~35 (both measured,
+// cache-resident table).  So everything that comes from global memory -- gathered rows, weight slabs,
+// neighbour indices -- is loaded in memory-friendly order straight into LDS (global_load_lds: no
+// registers, no masking; lanes without a neighbour read a row of zeros) and the MFMA operands are read
+// back from LDS.  With no staging registers the kernel fits 128 VGPRs, so two 8-wave workgroups (four
+// waves per SIMD, 512 output rows) share a CU and hide each other's latencies.
+// Hardware places lane l's bytes at base + 16 l, so the bank-conflict-free read order of the B operand is
+// obtained by permuting which chunk of its row a lane fetches: position p of a row holds chunk p ^ swz(row).
+//   iteration     = 4 K-steps = 4 KB of gathered rows per wave (32 rows x 8 chunks, or G = 8 / SEG
+//                   kernel offsets of SEG-chunk rows) and a weight slab of 4 * MT fragments
+//   LDS           = 2 weight slabs (iteration i, i+1), one 4 KB stage of gathered rows per wave, and a
+//                   4-deep ring of neighbour indices per wave (they always miss the caches)
+//   per iteration = one barrier for the slab; a wave consumes only rows and indices it fetched itself,
+//                   so those need a wait on the wave's own memory counter only
+// The memory counter retires loads in order, so "at most N outstanding" names exactly which older load
+// has landed.  Issue order per iteration i: slab S(i+1), indices I(i+4), gathers G(i+1).
+// waves per SIMD the kernel is compiled for: two 8-wave workgroups per CU, or one of 10 / 12 waves
+constexpr int conv_lds_min_waves(int waves) { return waves <= 8 ? 4 : 3; }
+
+template <int EL, int CHUNKS, int MT, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_lds(const ConvArgs a) {
+  using Acc = typename Mma32<EL>::Acc;
+  using Acc4 = typename Mma32<EL>::Acc4;
+  constexpr int THREADS = 64 * WAVES;
+  constexpr int SEG = CHUNKS < 8 ? CHUNKS : 8;   // chunks gathered per row and iteration
+  constexpr int IPO = CHUNKS / SEG;              // iterations per kernel offset (rows wider than 128 B)
+  constexpr int G = 8 / SEG;                     // kernel offsets per iteration
+  constexpr int RP = 8 / SEG;                    // rows per 128 bytes of the gathered stage
+  constexpr int SLAB = 4 * MT * 64;              // 16-byte weight fragments per iteration
+  constexpr int NL = SLAB / 64;                  // 1 KB wave-loads per slab
+  constexpr int WPT = (NL + WAVES - 1) / WAVES;  // slab loads per wave and iteration (the same for every wave:
+                                                 // the waits below count loads; surplus ones go to `spare`)
+  constexpr int IDXI = G >= 2 ? G / 2 : 1;       // index loads per wave and iteration (64 entries each)
+  constexpr int R = 32 * WAVES;                  // output rows per workgroup
+  __shared__ v4i lds[2][SLAB];
+  __shared__ v4i ring[WAVES][256];
+  __shared__ int32_t iring[4][WAVES][64 * IDXI];
+  __shared__ v4i spare[NL % WAVES ? 64 : 1];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int ln = lane & 31, lh = lane >> 5;
+  const uint32_t n = eff_n(a.n_out_dev, a.n_bound);
+  uint32_t tile;
+  if (!xcd_tile(n, R, &tile)) return;
+  const uint32_t row0 = (tile * WAVES + wave) * 32;
+  const int iters = IPO > 1 ? a.kvol * IPO : (a.kvol + G - 1) / G;
+  const char* __restrict__ xb = a.x;
+  const char* __restrict__ zrow = a.zrow;
+  const v4i* __restrict__ wsrc = reinterpret_cast<const v4i*>(a.wfrag);
+  const uint32_t ldb = a.x_ld_bytes;
+  const int32_t* __restrict__ minus1 = reinterpret_cast<const int32_t*>(a.zrow + 512);  // words of -1
+
+  Acc acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[t][j] = 0;
+
+  typedef const __attribute__((address_space(1))) void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+#define SCN_WAIT_VM(N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory")
+// LDS reads of what global_load_lds wrote are written in assembly: the compiler orders a visible LDS read
+// after EVERY outstanding global_load_lds (vmcnt(0)), which would drain the loads issued for the next
+// iterations.  The waits that are really needed are the explicit ones below.
+// weight slab of iteration IT -> LDS buffer IT % 2 (iterations past the end re-load the last slab)
+#define SCN_SLAB(IT)                                                                            \
+  {                                                                                             \
+    const int it_ = (IT) < iters ? (IT) : iters - 1;                                            \
+    _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                                           \
+      const int f_ = j * WAVES + wave; /* wave-uniform */                                       \
+      if (NL % WAVES == 0 || f_ < NL)                                                           \
+        __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + (size_t)it_ * SLAB + f_ * 64 + lane),  \
+                                         (lptr_t)&lds[(IT) & 1][f_ * 64], 16, 0, 0);            \
+      else                                                                                      \
+        __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + (size_t)it_ * SLAB + lane),            \
+                                         (lptr_t)&spare[0], 16, 0, 0);                          \
+    }                                                                                           \
+  }
+// neighbour rows of iteration IT -> index ring stage IT % 4: entry e = 64 q + lane is kernel offset
+// e / 32 of the iteration, tile row e % 32; slots outside the volume or beyond row n read -1
+#define SCN_INDEX(IT)                                                                           \
+  {                                                                                             \
+    _Pragma("unroll") for (int q = 0; q < IDXI; ++q) {                                          \
+      const int e_ = q * 64 + lane;                                                             \
+      const int k_ = IPO > 1 ? (IT) / IPO + e_ / 32 : (IT) * G + e_ / 32;                       \
+      const uint32_t r_ = row0 + (e_ & 31);                                                     \
+      const bool ok_ = (IT) < iters && k_ < a.kvol && r_ < n;                                   \
+      const int32_t* p_ = ok_ ? a.nbr + (size_t)k_ * a.nbr_ld + r_ : minus1 + lane;             \
+      __builtin_amdgcn_global_load_lds((gptr_t)p_, (lptr_t)&iring[(IT) & 3][wave][q * 64], 4, 0, 0); \
+    }                                                                                           \
+  }
+// gathers of iteration IT (neighbour rows GI[4] of this lane's slots) into the wave's stage; element
+// e = 64 q + lane of its [G][32 rows][SEG] array
+#define SCN_GATHER(IT, GI)                                                                      \
+  {                                                                                             \
+    _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                             \
+      const int e_ = q * 64 + lane;                                                             \
+      const int row_ = (e_ / SEG) % 32;                                                         \
+      const int cg_ = (IPO > 1 ? ((IT) % IPO) * 8 : 0) + ((e_ % SEG) ^ ((row_ / RP) % SEG));    \
+      const char* p_ = GI[q] >= 0 ? xb + (size_t)(uint32_t)GI[q] * ldb + cg_ * 16 : zrow + cg_ * 16; \
+      __builtin_amdgcn_global_load_lds((gptr_t)p_, (lptr_t)&ring[wave][q * 64], 16, 0, 0);      \
+    }                                                                                           \
+  }
+// this lane's four index slots of ring stage STG -> GI[4], waited for.  Slot q of lane l is entry
+// e / SEG of the stage (e = 64 q + l), i.e. a fixed stride of 64 / SEG entries between slots.
+#define SCN_READ_INDEX(STG, GI)                                                                 \
+  {                                                                                             \
+    const uint32_t base_ = iring_addr + (uint32_t)(STG) * (WAVES * 64 * IDXI * 4);              \
+    asm volatile("ds_read_b32 %0, %4\n\tds_read_b32 %1, %4 offset:%5\n\tds_read_b32 %2, %4 offset:%6\n\t" \
+                 "ds_read_b32 %3, %4 offset:%7\n\ts_waitcnt lgkmcnt(0)"                         \
+                 : "=&v"(GI[0]), "=&v"(GI[1]), "=&v"(GI[2]), "=&v"(GI[3])                       \
+                 : "v"(base_), "n"(256 / SEG), "n"(2 * 256 / SEG), "n"(3 * 256 / SEG)           \
+                 : "memory");                                                                   \
+  }
+// A fragments of K-step SS from the slab at LDS byte address LA (+ lane * 16 already included)
+#define SCN_READ_A(SS, LA, AF)                                                                  \
+  {                                                                                             \
+    if constexpr (MT == 4)                                                                      \
+      asm volatile("ds_read_b128 %0, %4 offset:%5\n\tds_read_b128 %1, %4 offset:%6\n\t"         \
+                   "ds_read_b128 %2, %4 offset:%7\n\tds_read_b128 %3, %4 offset:%8"             \
+                   : "=&v"(AF[0]), "=&v"(AF[1]), "=&v"(AF[2]), "=&v"(AF[3])                     \
+                   : "v"(LA), "n"(((SS) * 4 + 0) * 1024), "n"(((SS) * 4 + 1) * 1024),           \
+                     "n"(((SS) * 4 + 2) * 1024), "n"(((SS) * 4 + 3) * 1024)                     \
+                   : "memory");                                                                 \
+    else if constexpr (MT == 2)                                                                 \
+      asm volatile("ds_read_b128 %0, %2 offset:%3\n\tds_read_b128 %1, %2 offset:%4"             \
+                   : "=&v"(AF[0]), "=&v"(AF[1])                                                 \
+                   : "v"(LA), "n"(((SS) * 2 + 0) * 1024), "n"(((SS) * 2 + 1) * 1024)            \
+                   : "memory");                                                                 \
+    else                                                                                        \
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(AF[0]) : "v"(LA), "n"((SS) * 1024) : "memory"); \
+  }
+// wait until at most KEEP LDS operations are outstanding; AF is named as in/out so that its MFMAs stay below
+#define SCN_WAIT_A(KEEP, AF)                                                                    \
+  {                                                                                             \
+    if constexpr (MT == 4)                                                                      \
+      asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(AF[0]), "+v"(AF[1]), "+v"(AF[2]), "+v"(AF[3]) : "n"(KEEP) : "memory"); \
+    else if constexpr (MT == 2)                                                                 \
+      asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(AF[0]), "+v"(AF[1]) : "n"(KEEP) : "memory");  \
+    else                                                                                        \
+      asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(AF[0]) : "n"(KEEP) : "memory");               \
+  }
+
+  const uint32_t ring_addr = (uint32_t)(uintptr_t)(lptr_t)&ring[wave][0];
+  const uint32_t iring_addr = (uint32_t)(uintptr_t)(lptr_t)&iring[0][wave][0] + (uint32_t)(lane / SEG) * 4;
+  const uint32_t lds_a_addr = (uint32_t)(uintptr_t)(lptr_t)&lds[0][lane];
+  // B-operand read address of K-step ss inside the wave's stage: row ln, chunk 2 ss' + lh at its swizzled
+  // position.  Recomputed per iteration from two values (registers are what limits occupancy here).
+  const uint32_t b_base = ring_addr + (uint32_t)(SEG >= 2 ? ln * SEG : lh * 32 + ln) * 16;
+  const uint32_t b_swz = SEG >= 2 ? (uint32_t)(lh ^ ((ln / RP) % SEG)) : 0u;
+#define SCN_B_ADDR(SS, BB, SW)                                                                  \
+  (SEG >= 2 ? (BB) + (uint32_t)((((SS) / (SEG / 2 > 0 ? SEG / 2 : 1)) * 32 * SEG) +             \
+                                ((2 * ((SS) % (SEG / 2 > 0 ? SEG / 2 : 1))) ^ (SW))) * 16       \
+            : (BB) + (uint32_t)(2 * (SS) * 32) * 16)
+
+  // prologue: indices of iterations 0..3, slab 0, then the gathers of iteration 0
+  SCN_INDEX(0);
+  SCN_INDEX(1);
+  SCN_INDEX(2);
+  SCN_INDEX(3);
+  SCN_SLAB(0);
+  SCN_WAIT_VM(0);
+  {
+    int32_t gi[4];
+    SCN_READ_INDEX(0, gi);
+    SCN_GATHER(0, gi);
+  }
+  asm volatile("s_barrier" ::: "memory");
+
+  for (int it = 0; it < iters; ++it) {
+    SCN_SLAB(it + 1);
+    SCN_INDEX(it + 4);
+    SCN_WAIT_VM(WPT + IDXI);  // G(it), I(it+1) and everything older have landed
+    v4i bf[4];
+    int32_t gi[4];
+    {
+      uint32_t bb = b_base, sw = b_swz;
+      asm volatile("" : "+v"(bb), "+v"(sw));  // keeps the four addresses out of loop-carried registers
+      asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\tds_read_b128 %3, %7"
+                   : "=&v"(bf[0]), "=&v"(bf[1]), "=&v"(bf[2]), "=&v"(bf[3])
+                   : "v"(SCN_B_ADDR(0, bb, sw)), "v"(SCN_B_ADDR(1, bb, sw)), "v"(SCN_B_ADDR(2, bb, sw)),
+                     "v"(SCN_B_ADDR(3, bb, sw))
+                   : "memory");
+    }
+    // waits for the index reads and, LDS returning in order, for bf[]: the stage may be overwritten
+    SCN_READ_INDEX((it + 1) & 3, gi);
+    SCN_GATHER(it + 1, gi);
+    const uint32_t la = lds_a_addr + (uint32_t)(it & 1) * (SLAB * 16);
+    if constexpr (MT >= 4 && conv_lds_min_waves(WAVES) >= 4) {
+      // 64 accumulator registers leave room for one set of fragments under the 128-register budget of
+      // four waves per SIMD (a spill would also put scratch loads into the memory counter and break the
+      // counts above); the other three waves of the SIMD cover the LDS latency instead
+      v4i af[MT];
+#pragma unroll
+      for (int ss = 0; ss < 4; ++ss) {
+        SCN_READ_A(ss, la, af);
+        SCN_WAIT_A(0, af);
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[t] = Mma32<EL>::run(af[t], bf[ss], acc[t]);
+      }
+    } else {
+      v4i afA[MT], afB[MT];
+      SCN_READ_A(0, la, afA);
+      SCN_READ_A(1, la, afB);
+      SCN_WAIT_A(MT, afA);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = Mma32<EL>::run(afA[t], bf[0], acc[t]);
+      SCN_READ_A(2, la, afA);
+      SCN_WAIT_A(MT, afB);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = Mma32<EL>::run(afB[t], bf[1], acc[t]);
+      SCN_READ_A(3, la, afB);
+      SCN_WAIT_A(MT, afA);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = Mma32<EL>::run(afA[t], bf[2], acc[t]);
+      SCN_WAIT_A(0, afB);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = Mma32<EL>::run(afB[t], bf[3], acc[t]);
+    }
+    SCN_WAIT_VM(4);  // this wave's part of S(it+1) has landed (younger: G(it+1))
+    // every wave has read slab it (its fragments are in registers) and written its part of slab it+1
+    asm volatile("s_barrier" ::: "memory");
+  }
+#undef SCN_READ_INDEX
+#undef SCN_B_ADDR
+#undef SCN_READ_A
+#undef SCN_WAIT_A
+#undef SCN_WAIT_VM
+#undef SCN_SLAB
+#undef SCN_INDEX
+#undef SCN_GATHER
+  // Epilogue.  Each lane holds 4-channel pieces of one row; writing them directly would touch every
+  // 128-byte line of the tile 16 times.  The pieces go through the wave's LDS stage instead (same XOR
+  // placement as the gathers) and leave as 16 bytes per lane, 8 lanes per row.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stage still receives the gathers issued past the end
+  const uint32_t row = row0 + ln;
+  const int cout_pad = (a.cout + 15) & ~15;
+  if (!a.out_vec16) {
+    if (row >= n) return;
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int co = t * 32 + g * 8 + lh * 4;
+        if (co >= cout_pad) continue;
+        const Acc4 piece = {acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
+        epilogue_store<EL>(a, row, co, piece);
+      }
+    return;
+  }
+  char* stage = reinterpret_cast<char*>(&ring[wave][0]);
+  const bool out8 = a.out_dtype == SCN_DTYPE_INT8;
+  constexpr int PASSES = MT >= 4 ? 2 : 1;          // fp16 rows of 128 channels take two 128-byte passes
+  constexpr int TPP = MT >= 4 ? 2 : MT;            // 32-channel tiles per fp16 pass
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    if (out8 && p > 0) break;
+    const int t_lo = out8 ? 0 : p * TPP, t_hi = out8 ? MT : p * TPP + TPP;
+    const int c0 = t_lo * 32;                      // first channel of the pass
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      if (t < t_lo || t >= t_hi) continue;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int co = t * 32 + g * 8 + lh * 4;
+        if (co >= cout_pad || row >= n) continue;
+        const Acc4 piece = {acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
+        float y[4];
+        epilogue_values<EL>(a, row, co, piece, y);
+        const int off = (co - c0) * (out8 ? 1 : 2);  // byte offset inside the 128-byte pass row
+        char* dst = stage + ln * 128 + (((off >> 4) ^ (ln & 7)) << 4) + (off & 15);
+        if (out8)
+          *reinterpret_cast<char4*>(dst) = pack_int8(a, y);
+        else
+          *reinterpret_cast<v4h*>(dst) = pack_fp16(y);
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    const int osz = out8 ? 1 : 2;
+    const int valid = (cout_pad - c0) * osz;       // bytes of the pass row that exist
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int r = (lane >> 3) + 8 * j, c = lane & 7;
+      const uint32_t grow = row0 + r;
+      if (grow < n && c * 16 < valid) {
+        const v4i v = *reinterpret_cast<const v4i*>(stage + r * 128 + ((c ^ (r & 7)) << 4));
+        *reinterpret_cast<v4i*>(a.out + ((size_t)grow * a.out_ld + c0) * osz + c * 16) = v;
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+}
+
+// SCN_CONV_IMPL=rows forces the plain row-split kernel (A/B measurements; it is also the fallback for
+// more than 128 output channels).
+static int conv_impl() {
+  static const int impl = [] {
+    const char* e = getenv("SCN_CONV_IMPL");
+    return (e && !strcmp(e, "rows")) ? 1 : 0;
+  }();
+  return impl;
+}
+
+template <int EL, int CHUNKS, int MT>
+static void launch_conv_rows(const ConvArgs& a, hipStream_t stream) {
+  constexpr int NT = MT >= 8 ? 2 : 4;
+  const uint32_t rows_per_block = 4 * 16 * NT;
+  const uint32_t blocks = 8 * ceil_div(ceil_div(a.n_bound, rows_per_block), 8);  // see xcd_tile()
+  hipLaunchKernelGGL((k_conv_rows<EL, CHUNKS, MT, NT>), dim3(blocks), dim3(256), 0, stream, a);
+}
+
+template <int EL, int CHUNKS, int MT, int WAVES>
+static void launch_conv_lds(const ConvArgs& a, hipStream_t stream) {
+  constexpr uint32_t R = 32 * WAVES;
+  const uint32_t blocks = 8 * ceil_div(ceil_div(a.n_bound, R), 8);  // see xcd_tile()
+  hipLaunchKernelGGL((k_conv_lds<EL, CHUNKS, MT, WAVES>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
+}
+
+// Workgroup size of the 128-channel kernel.  A layer of a lidar backbone's deep stages is about one
+// workgroup per CU, so its duration is that of the busiest CU: 257 tiles of 256 rows on 256 CUs take
+// as long as 512.  With the expected row count (the count of the previous forward, see
+// Rulebook::n_out_hint) the tile height is chosen so that all rows fit one workgroup per CU when they
+// can: 8 to 12 waves of 32 rows; beyond 384 rows per CU it is 8 waves and two workgroups per CU.
+static int conv_lds_waves(uint32_t n_hint) {
+  static const int forced = [] {
+    const char* e = getenv("SCN_CONV_WAVES");
+    return e ? atoi(e) : 0;
+  }();
+  if (forced >= 8 && forced <= 12) return forced;
+  constexpr uint32_t kCus = 256;
+  const uint32_t waves = ceil_div(n_hint, kCus * 32u);  // 32-row tiles per CU
+  if (waves <= 8) return 8;
+  if (waves <= 12) return (int)waves;
+  return 8;
+}
+
+template <int EL, int CHUNKS>
+static bool dispatch_mt32(int mt, uint32_t n_hint, const ConvArgs& a, hipStream_t stream) {
+  switch (mt) {
+    case 1: launch_conv_lds<EL, CHUNKS, 1, 4>(a, stream); return true;
+    case 2: launch_conv_lds<EL, CHUNKS, 2, 8>(a, stream); return true;
+    case 4:
+      switch (conv_lds_waves(n_hint)) {
+        case 9: launch_conv_lds<EL, CHUNKS, 4, 9>(a, stream); return true;
+        case 10: launch_conv_lds<EL, CHUNKS, 4, 10>(a, stream); return true;
+        case 11: launch_conv_lds<EL, CHUNKS, 4, 11>(a, stream); return true;
+        case 12: launch_conv_lds<EL, CHUNKS, 4, 12>(a, stream); return true;
+        default: launch_conv_lds<EL, CHUNKS, 4, 8>(a, stream); return true;
+      }
+    default: return false;
+  }
+}
+
+template <int EL>
+static bool dispatch_chunks32(int chunks, int mt, uint32_t n_hint, const ConvArgs& a, hipStream_t stream) {
+  switch (chunks) {
+    case 1: return dispatch_mt32<EL, 1>(mt, n_hint, a, stream);
+    case 2: return dispatch_mt32<EL, 2>(mt, n_hint, a, stream);
+    case 4: return dispatch_mt32<EL, 4>(mt, n_hint, a, stream);
+    case 8: return dispatch_mt32<EL, 8>(mt, n_hint, a, stream);
+    case 16: return dispatch_mt32<EL, 16>(mt, n_hint, a, stream);
+    default: return false;
+  }
+}
+
+template <int EL, int CHUNKS>
+static bool dispatch_mt(int mt, const ConvArgs& a, hipStream_t stream) {
+  switch (mt) {
+    case 1: launch_conv_rows<EL, CHUNKS, 1>(a, stream); return true;
+    case 2: launch_conv_rows<EL, CHUNKS, 2>(a, stream); return true;
+    case 4: launch_conv_rows<EL, CHUNKS, 4>(a, stream); return true;
+    case 8: launch_conv_rows<EL, CHUNKS, 8>(a, stream); return true;
+    default: return false;
+  }
+}
+
+template <int EL>
+static bool dispatch_chunks(int chunks, int mt, const ConvArgs& a, hipStream_t stream) {
+  switch (chunks) {
+    case 1: return dispatch_mt<EL, 1>(mt, a, stream);
+    case 2: return dispatch_mt<EL, 2>(mt, a, stream);
+    case 4: return dispatch_mt<EL, 4>(mt, a, stream);
+    case 8: return dispatch_mt<EL, 8>(mt, a, stream);
+    case 16: return dispatch_mt<EL, 16>(mt, a, stream);
+    default: return false;
+  }
+}
+
+}  // namespace scn

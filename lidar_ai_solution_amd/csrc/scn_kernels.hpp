@@ -143,6 +143,14 @@ int permute_dense(const void* in, const int64_t in_shape[5], const int perm[5], 
 
 }  // namespace scn
 
+// Rulebook and convolution objects of the C ABI.
+struct scn_rulebook {
+  scn::Rulebook rb;
+};
+struct scn_conv {
+  scn::ConvWeights w;
+};
+
 // Voxelizer object of the C ABI.
 struct scn_voxelizer {
   scn_voxelization_param p{};
