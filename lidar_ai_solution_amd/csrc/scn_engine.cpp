@@ -1423,7 +1423,17 @@ static std::vector<int> attr_ints3(const OnnxNode& n, const char* name) {
 
 scn_engine* scn_engine_create_from_onnx(const char* onnx_file, int precision, unsigned flags,
                                         unsigned fixed_launch_points, void* stream) {
+  return scn_engine_create_from_onnx_ex(onnx_file, precision, flags, fixed_launch_points, nullptr, 0, stream);
+}
+
+scn_engine* scn_engine_create_from_onnx_ex(const char* onnx_file, int precision, unsigned flags,
+                                           unsigned fixed_launch_points, const scn_precision_override* overrides,
+                                           int n_overrides, void* stream) {
   if (!onnx_file) return nullptr;
+  if (n_overrides < 0 || (n_overrides > 0 && !overrides)) {
+    set_error("create_from_onnx: invalid precision overrides");
+    return nullptr;
+  }
   SCN_LOGV("Load onnx from: %s", onnx_file);
   std::ifstream fin(onnx_file, std::ios::binary);
   if (!fin) {
@@ -1472,9 +1482,22 @@ scn_engine* scn_engine_create_from_onnx(const char* onnx_file, int precision, un
     }
     return it->second;
   };
-  auto prec_of = [](const OnnxNode& n, const char* attr) {
+  // the node's own attribute unless an override names the node or its operator type (the last match wins)
+  auto prec_of = [&](const OnnxNode& n, const char* attr) {
     const OnnxAttr* a = n.find(attr);
-    return (a && a->s == "int8") ? SCN_PRECISION_INT8 : SCN_PRECISION_FP16;
+    int p = (a && a->s == "int8") ? SCN_PRECISION_INT8 : SCN_PRECISION_FP16;
+    const bool is_output = !strcmp(attr, "output_precision");
+    for (int i = 0; i < n_overrides; ++i) {
+      const scn_precision_override& o = overrides[i];
+      if (!o.selector) continue;
+      const std::string& subject = o.by_optype ? n.op_type : n.name;
+      const bool add_alias = o.by_optype && (n.op_type == "Add" || n.op_type == "QuantAdd") &&
+                             (!strcmp(o.selector, "Add") || !strcmp(o.selector, "QuantAdd"));
+      if (subject != o.selector && !add_alias) continue;
+      const int v = is_output ? o.output_precision : o.precision;
+      if (v == SCN_PRECISION_FP16 || v == SCN_PRECISION_INT8) p = v;
+    }
+    return p;
   };
   for (auto& n : g.nodes) {
     unsigned flp = fixed_launch_points;

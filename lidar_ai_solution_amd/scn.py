@@ -96,12 +96,25 @@ class Engine:
 
     @classmethod
     def from_onnx(cls, path: str, precision="fp16", sortmask=False, enable_blackwell=False, with_auxiliary_stream=False,
-                  fixed_launch_points: int = 10000, stream=None, keep_all: bool = False) -> "Engine":
-        """spconv::load_engine_from_onnx.  Raises instead of returning nullptr on failure."""
+                  fixed_launch_points: int = 10000, stream=None, keep_all: bool = False,
+                  precision_overrides=()) -> "Engine":
+        """spconv::load_engine_from_onnx.  Raises instead of returning nullptr on failure.
+
+        precision_overrides: (selector, by_optype, precision, output_precision) tuples applied to the
+        nodes' precisions before the engine is planned -- the older interface's set_node_precision_byname /
+        set_node_precision_byoptype + reconfigure; precision None leaves the model's value."""
         flags = (capi.BUILD_SORTMASK if sortmask else 0) | (capi.BUILD_AUX_STREAM if with_auxiliary_stream else 0) | \
                 (capi.BUILD_KEEP_ALL if keep_all else 0)
-        h = capi.lib().scn_engine_create_from_onnx(path.encode(), _prec(precision), flags, fixed_launch_points,
-                                                   _stream_ptr(stream) if stream is not None else None)
+        n = len(precision_overrides)
+        arr = (capi.PrecisionOverride * max(n, 1))()
+        for i, (sel, by_optype, prec, out_prec) in enumerate(precision_overrides):
+            arr[i].selector = sel.encode()
+            arr[i].by_optype = int(bool(by_optype))
+            arr[i].precision = _prec(prec) if prec is not None else 0
+            arr[i].output_precision = _prec(out_prec) if out_prec is not None else 0
+        h = capi.lib().scn_engine_create_from_onnx_ex(path.encode(), _prec(precision), flags, fixed_launch_points,
+                                                      C.cast(arr, C.c_void_p) if n else None, n,
+                                                      _stream_ptr(stream) if stream is not None else None)
         return cls(h)
 
     @classmethod

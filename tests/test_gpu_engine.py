@@ -429,3 +429,59 @@ def test_cpp_example_driver_matches_python_engine(cp_models, centerpoint_input, 
         got = tensor.load(prefix + ".0.tensor")
         assert got.shape == (1, 256, 180, 180) and got.dtype == np.float16
         assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+def test_legacy_single_call_interface_and_precision_overrides(cp_models, centerpoint_input, tmp_path):
+    """The older engine interface (forward(shapes, types, pointers, ...) -> DTensor*, set_node_precision_by*,
+    reconfigure) through the C++ caller built against include/legacy/spconv/engine.hpp, and the loader's
+    precision overrides through the Python mirror: the int8 model gives the int8 engine's bits; with every
+    node overridden to fp16 it gives the fp16 engine's bits; an override by node name equals the same edit
+    made in the model."""
+    import copy
+    import subprocess
+    from lidar_ai_solution_amd import tensor
+    feats, idx = centerpoint_input
+    g16, g8 = cp_models
+    model = str(tmp_path / "cp.int8.scn.onnx")
+    onnx_dialect.save(g8, model)
+    eng8 = Engine.from_onnx(model, "int8")
+    _run_engine(eng8, feats, idx, GRID_ZYX)
+    want8 = eng8.output(0).torch().cpu().numpy()
+    eng16 = Engine.from_graph(g16, "fp16")
+    _run_engine(eng16, feats, idx, GRID_ZYX)
+    want16 = eng16.output(0).torch().cpu().numpy()
+    note("precision overrides by operator type through the loader")
+    ov = [("SparseConvolution", True, "fp16", "fp16"), ("Add", True, "fp16", "fp16")]
+    eng = Engine.from_onnx(model, "int8", precision_overrides=ov)
+    _run_engine(eng, feats, idx, GRID_ZYX)
+    assert np.array_equal(eng.output(0).torch().cpu().numpy().view(np.uint16), want16.view(np.uint16))
+    note("override by node name == the same attribute edited in the model")
+    victim = [n for n in g8.nodes if n.op_type == "SparseConvolution"][10]
+    assert victim.attrs["precision"] == "int8"
+    g_edit = copy.deepcopy(g8)
+    for n in g_edit.nodes:
+        if n.name == victim.name:
+            n.attrs["precision"] = "fp16"
+    eng_a = Engine.from_onnx(model, "int8", precision_overrides=[(victim.name, False, "fp16", None)])
+    eng_b = Engine.from_graph(g_edit, "int8")
+    _run_engine(eng_a, feats, idx, GRID_ZYX)
+    _run_engine(eng_b, feats, idx, GRID_ZYX)
+    got_a = eng_a.output(0).torch().cpu().numpy()
+    assert np.array_equal(got_a.view(np.uint16), eng_b.output(0).torch().cpu().numpy().view(np.uint16))
+    assert not np.array_equal(got_a.view(np.uint16), want8.view(np.uint16))
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "lidar_ai_solution_amd", "examples",
+                       "infer_legacy")
+    if not os.path.exists(exe):
+        pytest.skip("legacy example driver not built (python -c 'import __graft_entry__ as g; g.build()')")
+    tensor.save(feats, str(tmp_path / "f.tensor"))
+    tensor.save(idx, str(tmp_path / "i.tensor"))
+    for extra, want in (([], want8), (["all-fp16"], want16)):
+        note(f"C++ caller of the legacy interface {extra}")
+        prefix = str(tmp_path / ("legacy" + "".join(extra)))
+        r = subprocess.run([exe, model, str(tmp_path / "f.tensor"), str(tmp_path / "i.tensor"), "41", "1440", "1440", "int8",
+                            prefix] + extra, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+        print(r.stdout)
+        assert r.returncode == 0, r.stdout
+        got = tensor.load(prefix + ".0.tensor")
+        assert got.shape == (1, 256, 180, 180) and got.dtype == np.float16
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
