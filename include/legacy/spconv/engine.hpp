@@ -4,9 +4,10 @@
 // method names and argument meaning, so a caller of that interface only changes its include path
 // (-I<this repository>/include/legacy) and links libscn_hip.so + the HIP runtime.
 //
-// Differences, all reported through the log: reconfigure() re-reads the model file with the precision
-// overrides collected so far (the engine is planned once per build); set_int8_calibration() is not available
-// in the engine -- dynamic ranges are calibrated offline and stored in the model file.
+// reconfigure() re-reads the model file with the precision overrides and the calibrated ranges collected so
+// far (the engine is planned once per build).  set_int8_calibration(true) switches to an fp16 engine that keeps
+// every tensor; each forward then records the largest magnitude of every tensor; set_int8_calibration(false)
+// + reconfigure() return to the requested precision with those ranges in place of the model's.
 #ifndef SCN_LEGACY_SPCONV_ENGINE_HPP
 #define SCN_LEGACY_SPCONV_ENGINE_HPP
 
@@ -99,6 +100,7 @@ class LegacyEngine : public Engine {
       fprintf(stderr, "[scn] forward failed: %s\n", scn_last_error());
       return nullptr;
     }
+    if (calibrating_) record_ranges(stream);
     scn_tensor_view v;
     if (scn_engine_output(e_, 0, &v) != SCN_OK) return nullptr;
     out_.assign(v);
@@ -108,9 +110,9 @@ class LegacyEngine : public Engine {
   void reconfigure() override { rebuild(); }
 
   void set_int8_calibration(bool enable) override {
-    if (enable)
-      fprintf(stderr, "[scn] set_int8_calibration: not available in the engine; calibrate offline and store the "
-                      "dynamic ranges in the model file\n");
+    if (enable == calibrating_) return;
+    calibrating_ = enable;
+    if (enable) rebuild();   // fp16, every tensor kept; leaving the mode takes effect at reconfigure()
   }
 
   void set_node_precision_byname(const char* name, Precision compute_precision, Precision output_precision) override {
@@ -127,12 +129,29 @@ class LegacyEngine : public Engine {
     selectors_.emplace_back(selector);
     pending_.push_back({by_optype, (int)c, (int)o});
   }
+  void record_ranges(void* stream) {
+    std::vector<scn_tensor_amax> got(4096);
+    const int n = scn_engine_collect_amax(e_, stream, got.data(), (int)got.size());
+    for (int i = 0; i < n; ++i) {
+      size_t j = 0;
+      while (j < range_names_.size() && range_names_[j] != got[i].tensor) ++j;
+      if (j == range_names_.size()) {
+        range_names_.emplace_back(got[i].tensor);
+        range_values_.push_back(0.f);
+      }
+      if (got[i].amax > range_values_[j]) range_values_[j] = got[i].amax;
+    }
+  }
   void rebuild() {
     std::vector<scn_precision_override> ov(pending_.size());
     for (size_t i = 0; i < pending_.size(); ++i)
       ov[i] = {selectors_[i].c_str(), pending_[i].by_optype, pending_[i].precision, pending_[i].output_precision};
-    scn_engine* fresh = scn_engine_create_from_onnx_ex(file_.c_str(), (int)precision_, 0u, 10000u,
-                                                       ov.empty() ? nullptr : ov.data(), (int)ov.size(), nullptr);
+    std::vector<scn_tensor_amax> rg(calibrating_ ? 0 : range_names_.size());
+    for (size_t i = 0; i < rg.size(); ++i) rg[i] = {range_names_[i].c_str(), range_values_[i]};
+    scn_load_options opt = {ov.empty() ? nullptr : ov.data(), (int)ov.size(), rg.empty() ? nullptr : rg.data(),
+                            (int)rg.size()};
+    scn_engine* fresh = scn_engine_create_from_onnx_ex(file_.c_str(), calibrating_ ? (int)Precision::Float16 : (int)precision_,
+                                                       calibrating_ ? SCN_BUILD_KEEP_ALL : 0u, 10000u, &opt, nullptr);
     if (!fresh) {
       fprintf(stderr, "[scn] load_engine_from_onnx(%s) failed: %s\n", file_.c_str(), scn_last_error());
       return;  // keeps the previous engine, if any
@@ -147,6 +166,9 @@ class LegacyEngine : public Engine {
   Precision precision_;
   std::vector<std::string> selectors_;
   std::vector<Pending> pending_;
+  std::vector<std::string> range_names_;
+  std::vector<float> range_values_;
+  bool calibrating_ = false;
   scn_engine* e_ = nullptr;
   OutputView out_;
 };

@@ -27,6 +27,14 @@ class PrecisionOverride(C.Structure):
     _fields_ = [("selector", C.c_char_p), ("by_optype", C.c_int), ("precision", C.c_int), ("output_precision", C.c_int)]
 
 
+class TensorAmax(C.Structure):
+    _fields_ = [("tensor", C.c_char_p), ("amax", C.c_float)]
+
+
+class LoadOptions(C.Structure):
+    _fields_ = [("overrides", C.c_void_p), ("n_overrides", C.c_int), ("ranges", C.c_void_p), ("n_ranges", C.c_int)]
+
+
 class VoxelizationParam(C.Structure):
     _fields_ = [("min_range", C.c_float * 3), ("max_range", C.c_float * 3), ("voxel_size", C.c_float * 3),
                 ("grid_size", C.c_int * 3), ("num_feature", C.c_int), ("max_voxels", C.c_int),
@@ -106,7 +114,8 @@ _SIGNATURES = {
     "scn_builder_push_output": (C.c_int, [vp, C.c_int]),
     "scn_builder_build": (vp, [vp, C.c_int, C.c_uint, vp]),
     "scn_engine_create_from_onnx": (vp, [C.c_char_p, C.c_int, C.c_uint, C.c_uint, vp]),
-    "scn_engine_create_from_onnx_ex": (vp, [C.c_char_p, C.c_int, C.c_uint, C.c_uint, vp, C.c_int, vp]),
+    "scn_engine_create_from_onnx_ex": (vp, [C.c_char_p, C.c_int, C.c_uint, C.c_uint, vp, vp]),
+    "scn_engine_collect_amax": (C.c_int, [vp, vp, vp, C.c_int]),
     "scn_engine_destroy": (None, [vp]),
     "scn_engine_num_input": (C.c_int, [vp]),
     "scn_engine_num_output": (C.c_int, [vp]),

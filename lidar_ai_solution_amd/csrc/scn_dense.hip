@@ -89,6 +89,39 @@ int add_relu(const void* a, int a_dtype, float a_range, float a_rq, const void* 
   return SCN_OK;
 }
 
+// max |value| over the first n rows x c channels of a row-major tensor (calibration: the dynamic range of a
+// tensor is the largest magnitude seen).  Non-negative floats order like their bit patterns, so the
+// reduction is an integer atomicMax; *result must be zero on entry.
+__global__ __launch_bounds__(256) void k_absmax(const void* x, int dtype, float scale, uint32_t c, uint32_t ld,
+                                               uint32_t n_bound, const uint32_t* n_dev, uint32_t* result) {
+  const uint32_t n = eff_n(n_dev, n_bound);
+  const size_t total = (size_t)n * c;
+  float m = 0.f;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+    const size_t row = i / c, col = i % c;
+    const float v = fabsf(load_value(x, dtype, row * ld + col, scale, 0.f, 0.f));
+    m = v > m ? v : m;   // NaN never wins
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, __shfl_xor(m, d, 64));
+  if ((threadIdx.x & 63) == 0 && m > 0.f) atomicMax(result, __float_as_uint(m));
+}
+
+int absmax_rows(const void* x, int dtype, float range, uint32_t c, uint32_t ld, uint32_t n, const uint32_t* n_dev,
+                float* result_dev, hipStream_t stream) {
+  SCN_REQUIRE(result_dev, SCN_ERR_INVALID, "absmax: null result");
+  int rc = fill_u32(result_dev, 0u, 1, stream);   // one word; the pointer must be 16-byte aligned
+  if (rc) return rc;
+  if (n == 0 || c == 0) return SCN_OK;
+  SCN_REQUIRE(x, SCN_ERR_INVALID, "absmax: null tensor");
+  const size_t total = (size_t)n * c;
+  const unsigned blocks = (unsigned)std::min<size_t>((total + 255) / 256, 2048);
+  hipLaunchKernelGGL(k_absmax, dim3(blocks), dim3(256), 0, stream, x, dtype, range > 0.f ? range / 127.f : 1.f, c, ld, n,
+                     n_dev, reinterpret_cast<uint32_t*>(result_dev));
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
 // --------------------------------------------------------------------------------------------
 // sparse -> dense.  strides are those of the final (possibly transposed) layout, in elements.
 // --------------------------------------------------------------------------------------------

@@ -180,6 +180,7 @@ struct scn_engine {
   std::vector<std::unique_ptr<ConvWeights>> convs;
   std::vector<Step> steps;
   std::vector<char> dense_precleared;  // per step: the forward's batched fill zeroed its dense output (1) or reset its row map (2)
+  DevBuf amax_buf;                     // collect_amax: one 16-byte slot per tensor
   bool dense_map_built = false;        // the step about to run had its row map built on the auxiliary stream
   hipEvent_t ev_map = nullptr;
   std::vector<DevBuf> dense_maps;      // per step: cell -> row map of a ScatterDense whose layout allows the dense-major pass
@@ -1423,17 +1424,28 @@ static std::vector<int> attr_ints3(const OnnxNode& n, const char* name) {
 
 scn_engine* scn_engine_create_from_onnx(const char* onnx_file, int precision, unsigned flags,
                                         unsigned fixed_launch_points, void* stream) {
-  return scn_engine_create_from_onnx_ex(onnx_file, precision, flags, fixed_launch_points, nullptr, 0, stream);
+  return scn_engine_create_from_onnx_ex(onnx_file, precision, flags, fixed_launch_points, nullptr, stream);
 }
 
 scn_engine* scn_engine_create_from_onnx_ex(const char* onnx_file, int precision, unsigned flags,
-                                           unsigned fixed_launch_points, const scn_precision_override* overrides,
-                                           int n_overrides, void* stream) {
+                                           unsigned fixed_launch_points, const scn_load_options* options,
+                                           void* stream) {
   if (!onnx_file) return nullptr;
-  if (n_overrides < 0 || (n_overrides > 0 && !overrides)) {
-    set_error("create_from_onnx: invalid precision overrides");
+  const scn_precision_override* overrides = options ? options->overrides : nullptr;
+  const int n_overrides = options ? options->n_overrides : 0;
+  const scn_tensor_amax* ranges = options ? options->ranges : nullptr;
+  const int n_ranges = options ? options->n_ranges : 0;
+  if (n_overrides < 0 || (n_overrides > 0 && !overrides) || n_ranges < 0 || (n_ranges > 0 && !ranges)) {
+    set_error("create_from_onnx: invalid load options");
     return nullptr;
   }
+  // calibrated |max| of a tensor, or 0 when the options hold none for it
+  auto range_of = [&](const std::string& tensor) {
+    float r = 0.f;
+    for (int i = 0; i < n_ranges; ++i)
+      if (ranges[i].tensor && tensor == ranges[i].tensor) r = ranges[i].amax;
+    return r;
+  };
   SCN_LOGV("Load onnx from: %s", onnx_file);
   std::ifstream fin(onnx_file, std::ios::binary);
   if (!fin) {
@@ -1519,6 +1531,13 @@ scn_engine* scn_engine_create_from_onnx_ex(const char* onnx_file, int precision,
       }
       std::vector<float> wr;
       if (const OnnxAttr* a = n.find("weight_dynamic_ranges")) wr = a->floats;
+      if (wr.empty() && n_ranges > 0) {
+        // calibration supplies activation ranges only: per-output-channel |max| of the weights, as the
+        // exporter writes them
+        const size_t per = w.size() / (size_t)wshape[0];
+        wr.assign((size_t)wshape[0], 0.f);
+        for (size_t i = 0; i < w.size(); ++i) wr[i / per] = std::max(wr[i / per], std::fabs(half_bits_to_float(w[i])));
+      }
       unsigned bound = 150000;
       if (const OnnxAttr* a = n.find("output_bound")) bound = (unsigned)a->i;
       else SCN_LOGV("using default output_bound: %u", bound);
@@ -1536,7 +1555,8 @@ scn_engine* scn_engine_create_from_onnx_ex(const char* onnx_file, int precision,
       out = scn_builder_push_sparse_conv(
           b.get(), n.name.c_str(), x, w.data(), wshape.data(), wr.empty() ? nullptr : wr.data(), (int)wr.size(),
           bias.data(), (int)bias.size(), act ? act->s.c_str() : "", ks.data(), st.size() == 3 ? st.data() : nullptr,
-          pd.size() == 3 ? pd.data() : nullptr, dl.size() == 3 ? dl.data() : nullptr, idr ? idr->f : 0.f,
+          pd.size() == 3 ? pd.data() : nullptr, dl.size() == 3 ? dl.data() : nullptr,
+          range_of(n.input[0]) > 0.f ? range_of(n.input[0]) : (idr ? idr->f : 0.f),
           subm ? (int)subm->i : 0, bound, flp, rb ? rb->s.c_str() : "", prec_of(n, "precision"),
           prec_of(n, "output_precision"), n.output[0].c_str(), inv ? (int)inv->i : 0);
     } else if (n.op_type == "Add" || n.op_type == "QuantAdd") {
@@ -1548,7 +1568,11 @@ scn_engine* scn_engine_create_from_onnx_ex(const char* onnx_file, int precision,
       if (a < 0 || c < 0) return nullptr;
       const OnnxAttr* r0 = n.find("input0_dynamic_range");
       const OnnxAttr* r1 = n.find("input1_dynamic_range");
-      out = scn_builder_push_add(b.get(), n.name.c_str(), a, c, r0 ? r0->f : 0.f, r1 ? r1->f : 0.f, n.output[0].c_str(),
+      float ra = r0 ? r0->f : 0.f, rb = r1 ? r1->f : 0.f;
+      // calibrated: one shared range for both operands, the larger of the two (what the exporter writes)
+      const float shared = std::max(range_of(n.input[0]), range_of(n.input[1]));
+      if (shared > 0.f) ra = rb = shared;
+      out = scn_builder_push_add(b.get(), n.name.c_str(), a, c, ra, rb, n.output[0].c_str(),
                                  prec_of(n, "precision"), prec_of(n, "output_precision"), fixed_launch_points);
     } else if (n.op_type == "Relu") {
       const int x = n.input.empty() ? -1 : tensor_of(n.input[0]);
@@ -1748,6 +1772,48 @@ int scn_engine_tensor(scn_engine* e, const char* name, scn_tensor_view* view, vo
   fill_view(e, it->second, view);
   if (acc_dev) *acc_dev = e->tensors[it->second].acc.p;
   return SCN_OK;
+}
+
+int scn_engine_collect_amax(scn_engine* e, void* stream_, scn_tensor_amax* out, int capacity) {
+  if (!e || !out || capacity < 0) {
+    set_error("collect_amax: invalid arguments");
+    return -1;
+  }
+  hipStream_t stream = (hipStream_t)stream_;
+  std::vector<int> which;
+  for (size_t t = 0; t < e->tdesc.size() && t < e->tensors.size(); ++t) {
+    const RtTensor& x = e->tensors[t];
+    if (x.dense || x.coord < 0 || !x.materialised) continue;
+    if ((int)t == e->inputs[0] ? e->in_feat == nullptr : x.data == nullptr) continue;
+    which.push_back((int)t);
+  }
+  if ((int)which.size() > capacity) {
+    set_error("collect_amax: %zu tensors, room for %d", which.size(), capacity);
+    return -1;
+  }
+  if (which.empty()) return 0;
+  if (e->amax_buf.bytes < which.size() * 16 && !e->amax_buf.alloc(which.size() * 16)) return -1;
+  for (size_t i = 0; i < which.size(); ++i) {
+    const int t = which[i];
+    const RtTensor& x = e->tensors[t];
+    const CoordSet& cs = e->coords[x.coord];
+    const bool is_input = t == e->inputs[0];
+    const int rc = absmax_rows(is_input ? e->in_feat : x.data, is_input ? SCN_DTYPE_FP16 : x.dtype, x.range,
+                               (uint32_t)(is_input ? e->in_c : x.c), is_input ? e->in_c : x.ld, cs.n_bound, cs.n_dev,
+                               reinterpret_cast<float*>(e->amax_buf.as<char>() + i * 16), stream);
+    if (rc) return -1;
+  }
+  std::vector<float> host(which.size() * 4);
+  if (hipMemcpyAsync(host.data(), e->amax_buf.p, which.size() * 16, hipMemcpyDeviceToHost, stream) != hipSuccess ||
+      hipStreamSynchronize(stream) != hipSuccess) {
+    set_error("collect_amax: copy failed");
+    return -1;
+  }
+  for (size_t i = 0; i < which.size(); ++i) {
+    out[i].tensor = e->tdesc[which[i]].name.c_str();
+    out[i].amax = host[i * 4];
+  }
+  return (int)which.size();
 }
 
 int scn_engine_set_profiling(scn_engine* e, int enabled) {

@@ -127,6 +127,9 @@ int convert_rows(const void* in, int in_dtype, uint32_t in_c, uint32_t in_ld, fl
 int add_relu(const void* a, int a_dtype, float a_range, float a_rq, const void* b, int b_dtype, float b_range,
              float b_rq, void* out, int out_dtype, float out_range, int relu, uint32_t c, uint32_t n,
              const uint32_t* n_dev, hipStream_t stream);
+// max |value| of the first min(*n_dev, n) rows x c channels -> *result_dev (a 16-byte aligned device float)
+int absmax_rows(const void* x, int dtype, float range, uint32_t c, uint32_t ld, uint32_t n, const uint32_t* n_dev,
+                float* result_dev, hipStream_t stream);
 int scatter_dense(const void* feat, int dtype, float range, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
                   const uint32_t* n_dev, const int dense_shape[5], const int perm[5], void* out, hipStream_t stream,
                   bool precleared = false, int32_t* cell_map = nullptr, bool map_precleared = false,

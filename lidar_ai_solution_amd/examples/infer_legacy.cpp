@@ -3,7 +3,7 @@
 // takes shapes, types and device pointers and returns the dense BEV tensor -- plus the precision overrides
 // of that interface.
 //
-//   infer_legacy <model.scn.onnx> <features.tensor> <indices.tensor> <g0> <g1> <g2> [fp16|int8] [output prefix] [all-fp16]
+//   infer_legacy <model.scn.onnx> <features.tensor> <indices.tensor> <g0> <g1> <g2> [fp16|int8] [output prefix] [all-fp16|calibrate]
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
@@ -16,12 +16,13 @@
 
 int main(int argc, char** argv) {
   if (argc < 7) {
-    printf("usage: %s model.onnx features.tensor indices.tensor g0 g1 g2 [fp16|int8] [output prefix] [all-fp16]\n", argv[0]);
+    printf("usage: %s model.onnx features.tensor indices.tensor g0 g1 g2 [fp16|int8] [output prefix] [all-fp16|calibrate]\n", argv[0]);
     return 1;
   }
   const auto precision = (argc > 7 && !strcmp(argv[7], "int8")) ? spconv::Precision::Int8 : spconv::Precision::Float16;
   const std::string out_prefix = argc > 8 ? argv[8] : "output";
   const bool all_fp16 = argc > 9 && !strcmp(argv[9], "all-fp16");
+  const bool calibrate = argc > 9 && !strcmp(argv[9], "calibrate");
   const std::vector<int> grid = {atoi(argv[4]), atoi(argv[5]), atoi(argv[6])};
   hipStream_t stream;
   if (hipStreamCreateWithFlags(&stream, hipStreamNonBlocking) != hipSuccess) return 2;
@@ -42,6 +43,18 @@ int main(int argc, char** argv) {
   if (features.empty() || indices.empty()) {
     printf("Failed to load the input tensors\n");
     return 4;
+  }
+  if (calibrate) {
+    // implicit calibration: one forward records every tensor's largest magnitude, then every convolution and
+    // Add is switched to int8 and the engine is planned again with those ranges
+    engine->set_int8_calibration(true);
+    if (engine->forward({features.size(0), features.size(1)}, spconv::DType::Float16, features.ptr(),
+                        {indices.size(0), indices.size(1)}, spconv::DType::Int32, indices.ptr(), 1, grid, stream) == nullptr)
+      return 5;
+    engine->set_int8_calibration(false);
+    engine->set_node_precision_byoptype("SparseConvolution", spconv::Precision::Int8, spconv::Precision::Int8);
+    engine->set_node_precision_byoptype("Add", spconv::Precision::Int8, spconv::Precision::Int8);
+    engine->reconfigure();
   }
   spconv::DTensor* result = nullptr;
   for (int rep = 0; rep < 2; ++rep)   // the second call re-uses everything the first one allocated

@@ -97,12 +97,14 @@ class Engine:
     @classmethod
     def from_onnx(cls, path: str, precision="fp16", sortmask=False, enable_blackwell=False, with_auxiliary_stream=False,
                   fixed_launch_points: int = 10000, stream=None, keep_all: bool = False,
-                  precision_overrides=()) -> "Engine":
+                  precision_overrides=(), tensor_ranges=None) -> "Engine":
         """spconv::load_engine_from_onnx.  Raises instead of returning nullptr on failure.
 
         precision_overrides: (selector, by_optype, precision, output_precision) tuples applied to the
         nodes' precisions before the engine is planned -- the older interface's set_node_precision_byname /
-        set_node_precision_byoptype + reconfigure; precision None leaves the model's value."""
+        set_node_precision_byoptype + reconfigure; precision None leaves the model's value.
+        tensor_ranges: {tensor name: calibrated |max|} (see collect_amax); replaces the dynamic ranges of the
+        model's convolutions and Adds."""
         flags = (capi.BUILD_SORTMASK if sortmask else 0) | (capi.BUILD_AUX_STREAM if with_auxiliary_stream else 0) | \
                 (capi.BUILD_KEEP_ALL if keep_all else 0)
         n = len(precision_overrides)
@@ -112,9 +114,15 @@ class Engine:
             arr[i].by_optype = int(bool(by_optype))
             arr[i].precision = _prec(prec) if prec is not None else 0
             arr[i].output_precision = _prec(out_prec) if out_prec is not None else 0
+        ranges = list((tensor_ranges or {}).items())
+        rarr = (capi.TensorAmax * max(len(ranges), 1))()
+        for i, (name, amax) in enumerate(ranges):
+            rarr[i].tensor = name.encode()
+            rarr[i].amax = float(amax)
+        opt = capi.LoadOptions(C.cast(arr, C.c_void_p) if n else None, n,
+                               C.cast(rarr, C.c_void_p) if ranges else None, len(ranges))
         h = capi.lib().scn_engine_create_from_onnx_ex(path.encode(), _prec(precision), flags, fixed_launch_points,
-                                                      C.cast(arr, C.c_void_p) if n else None, n,
-                                                      _stream_ptr(stream) if stream is not None else None)
+                                                      C.byref(opt), _stream_ptr(stream) if stream is not None else None)
         return cls(h)
 
     @classmethod
@@ -208,6 +216,15 @@ class Engine:
 
     def forward(self, stream=None):
         capi.check(capi.lib().scn_engine_forward(self._h, _stream_ptr(stream)))
+
+    def collect_amax(self, stream=None) -> Dict[str, float]:
+        """max |value| of every sparse tensor the engine holds after a forward (all of them with keep_all)."""
+        cap = 4096
+        arr = (capi.TensorAmax * cap)()
+        n = capi.lib().scn_engine_collect_amax(self._h, _stream_ptr(stream), C.cast(arr, C.c_void_p), cap)
+        if n < 0:
+            raise RuntimeError("collect_amax failed: " + capi.lib().scn_last_error().decode())
+        return {arr[i].tensor.decode(): float(arr[i].amax) for i in range(n)}
 
     def output(self, index: int = 0) -> TensorView:
         v = capi.TensorView()

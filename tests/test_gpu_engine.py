@@ -485,3 +485,58 @@ def test_legacy_single_call_interface_and_precision_overrides(cp_models, centerp
         got = tensor.load(prefix + ".0.tensor")
         assert got.shape == (1, 256, 180, 180) and got.dtype == np.float16
         assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+def test_implicit_calibration_collect_amax_and_ranges(cp_models, centerpoint_input, tmp_path):
+    """Implicit PTQ calibration of the older interface: the engine reports every tensor's largest magnitude
+    (equal to numpy's on the tensors read back), and a model without any ranges loaded with those ranges and
+    int8 overrides gives, bit for bit, what the same model annotated in Python (exporter rules) gives -- through
+    the Python mirror and through the C++ caller of the legacy header."""
+    import subprocess
+    from lidar_ai_solution_amd import tensor
+    feats, idx = centerpoint_input
+    n = 40000
+    feats, idx = feats[:n], idx[:n]
+    g16, _ = cp_models
+    model = str(tmp_path / "cp.fp16.scn.onnx")
+    onnx_dialect.save(g16, model)
+    note("collect_amax on an fp16 engine that keeps every tensor")
+    cal = Engine.from_onnx(model, "fp16", keep_all=True)
+    _run_engine(cal, feats, idx, GRID_ZYX)
+    amax = cal.collect_amax()
+    sparse_nodes = [nd for nd in g16.nodes if nd.op_type in ("SparseConvolution", "Add", "Relu")]
+    assert len(amax) == len(sparse_nodes) + 1
+    assert np.float32(amax[g16.inputs[0]]) == np.abs(feats.astype(np.float32)).max()
+    for nd in sparse_nodes:
+        view, _ = cal.tensor(nd.outputs[0])
+        f, _ = view.torch()
+        c = [x for x in g16.nodes if x.outputs[0] == nd.outputs[0]][0]
+        width = int(c.attrs["out_channels"]) if c.op_type == "SparseConvolution" else f.shape[1]
+        assert np.float32(amax[nd.outputs[0]]) == np.abs(f.cpu().numpy()[:, :width].astype(np.float32)).max(), nd.name
+    note("model without ranges + collected ranges + int8 overrides == the model annotated by the exporter's rules")
+    ov = [("SparseConvolution", True, "int8", "int8"), ("Add", True, "int8", "int8")]
+    eng = Engine.from_onnx(model, "int8", precision_overrides=ov, tensor_ranges=amax)
+    _run_engine(eng, feats, idx, GRID_ZYX)
+    got = eng.output(0).torch().cpu().numpy()
+    g8, tags8 = graphs.centerpoint_scn(seed=0)
+    graphs.apply_int8_plan(g8, tags8, amax, "all-int8")
+    ref_eng = Engine.from_graph(g8, "int8")
+    _run_engine(ref_eng, feats, idx, GRID_ZYX)
+    want = ref_eng.output(0).torch().cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16)) and np.count_nonzero(want) > 50000
+    oracle = O.run_graph(g8, feats, idx, GRID_ZYX, "int8")[g8.outputs[0]]
+    assert np.array_equal(want.view(np.uint16), oracle.view(np.uint16))
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "lidar_ai_solution_amd", "examples",
+                       "infer_legacy")
+    if not os.path.exists(exe):
+        pytest.skip("legacy example driver not built (python -c 'import __graft_entry__ as g; g.build()')")
+    note("C++ caller: set_int8_calibration(true), forward, set_int8_calibration(false), overrides, reconfigure")
+    tensor.save(feats, str(tmp_path / "f.tensor"))
+    tensor.save(idx, str(tmp_path / "i.tensor"))
+    prefix = str(tmp_path / "calibrated")
+    r = subprocess.run([exe, model, str(tmp_path / "f.tensor"), str(tmp_path / "i.tensor"), "41", "1440", "1440", "int8",
+                        prefix, "calibrate"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    print(r.stdout)
+    assert r.returncode == 0, r.stdout
+    out = tensor.load(prefix + ".0.tensor")
+    assert np.array_equal(out.view(np.uint16), want.view(np.uint16))
