@@ -305,7 +305,8 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
   constexpr int R = 32 * WAVES;                  // output rows per workgroup
   __shared__ v4i lds[2][SLAB];
   __shared__ v4i ring[WAVES][256];
-  __shared__ int32_t iring[4][WAVES][64 * IDXI];
+  constexpr int DEPTH = (MT == 1 && CHUNKS <= 2) ? 2 : 4;   // index ring stages (LDS is what limits the narrow layers' occupancy)
+  __shared__ int32_t iring[DEPTH][WAVES][64 * IDXI];
   __shared__ v4i spare[NL % WAVES ? 64 : 1];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -357,7 +358,7 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
       const uint32_t r_ = row0 + (e_ & 31);                                                     \
       const bool ok_ = (IT) < iters && k_ < a.kvol && r_ < n;                                   \
       const int32_t* p_ = ok_ ? a.nbr + (size_t)k_ * a.nbr_ld + r_ : minus1 + lane;             \
-      __builtin_amdgcn_global_load_lds((gptr_t)p_, (lptr_t)&iring[(IT) & 3][wave][q * 64], 4, 0, 0); \
+      __builtin_amdgcn_global_load_lds((gptr_t)p_, (lptr_t)&iring[(IT) & (DEPTH - 1)][wave][q * 64], 4, 0, 0); \
     }                                                                                           \
   }
 // gathers of iteration IT (neighbour rows GI[4] of this lane's slots) into the wave's stage; element
@@ -427,8 +428,10 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
   // prologue: indices of iterations 0..3, slab 0, then the gathers of iteration 0
   SCN_INDEX(0);
   SCN_INDEX(1);
-  SCN_INDEX(2);
-  SCN_INDEX(3);
+  if constexpr (DEPTH == 4) {
+    SCN_INDEX(2);
+    SCN_INDEX(3);
+  }
   SCN_SLAB(0);
   SCN_WAIT_VM(0);
   {
@@ -440,7 +443,7 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
 
   for (int it = 0; it < iters; ++it) {
     SCN_SLAB(it + 1);
-    SCN_INDEX(it + 4);
+    SCN_INDEX(it + DEPTH);
     SCN_WAIT_VM(WPT + IDXI);  // G(it), I(it+1) and everything older have landed
     v4i bf[4];
     int32_t gi[4];
@@ -454,7 +457,7 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
                    : "memory");
     }
     // waits for the index reads and, LDS returning in order, for bf[]: the stage may be overwritten
-    SCN_READ_INDEX((it + 1) & 3, gi);
+    SCN_READ_INDEX((it + 1) & (DEPTH - 1), gi);
     SCN_GATHER(it + 1, gi);
     const uint32_t la = lds_a_addr + (uint32_t)(it & 1) * (SLAB * 16);
     if constexpr (MT >= 4 && conv_lds_min_waves(WAVES) >= 4) {
