@@ -182,7 +182,6 @@ struct scn_engine {
   std::vector<char> dense_precleared;  // per step: the forward's batched fill zeroed its dense output (1) or reset its row map (2)
   DevBuf amax_buf;                     // collect_amax: one 16-byte slot per tensor
   bool dense_map_built = false;        // the step about to run had its row map built on the auxiliary stream
-  hipEvent_t ev_map = nullptr;
   std::vector<DevBuf> dense_maps;      // per step: cell -> row map of a ScatterDense whose layout allows the dense-major pass
   std::map<std::string, int> tensor_by_name;
   // input binding
@@ -204,6 +203,7 @@ struct scn_engine {
   std::vector<hipEvent_t> rb_ready;   // per rulebook
   std::vector<int> rb_seq;            // per rulebook: position in the auxiliary stream's order (this forward)
   std::vector<int> coord_rb;          // per coordinate set: rulebook that produced it (-1: graph input)
+  std::vector<char> map_built;        // per step: the dense output's row map was built on the auxiliary stream
   ~scn_engine() {
     for (auto& s : steps) {
       if (s.ev0) (void)hipEventDestroy(s.ev0);
@@ -213,7 +213,6 @@ struct scn_engine {
       if (ev) (void)hipEventDestroy(ev);
     if (ev_fork) (void)hipEventDestroy(ev_fork);
     if (ev_join) (void)hipEventDestroy(ev_join);
-    if (ev_map) (void)hipEventDestroy(ev_map);
     if (aux) (void)hipStreamDestroy(aux);
   }
 };
@@ -857,7 +856,6 @@ static int allocate_runtime(scn_engine& e) {
     SCN_HIP(hipStreamCreateWithFlags(&e.aux, hipStreamNonBlocking));  // default priority
     SCN_HIP(hipEventCreateWithFlags(&e.ev_fork, hipEventDisableTiming));
     SCN_HIP(hipEventCreateWithFlags(&e.ev_join, hipEventDisableTiming));
-    SCN_HIP(hipEventCreateWithFlags(&e.ev_map, hipEventDisableTiming));
     e.rb_ready.assign(e.rulebooks.size(), nullptr);
     for (auto& ev : e.rb_ready) SCN_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
   }
@@ -1657,13 +1655,78 @@ int scn_engine_forward(scn_engine* e, void* stream_) {
     int rc = allocate_runtime(*e);
     if (rc) return rc;
   }
-  // Two streams unless per-step profiling is on.  The auxiliary stream is in order, so waiting for a
-  // rulebook's event also covers everything built before it.
+  // Two streams unless per-step profiling is on.  Coordinate work (hash, rulebooks, row maps of the
+  // dense outputs) depends on the input coordinates alone, so all of it is enqueued on the auxiliary
+  // stream first, in graph order, and runs as far ahead of the feature kernels as the GPU allows; the
+  // main stream then waits per rulebook.  The auxiliary stream is in order, so waiting for a rulebook's
+  // event also covers everything built before it.
   const bool dual = e->aux != nullptr && !e->profiling;
-  int aux_seq = 0, waited_seq = 0;
+  auto is_coord_step = [](const Step& st) {
+    return st.kind == StepKind::HashBuild || st.kind == StepKind::RulebookSubm || st.kind == StepKind::RulebookSparse ||
+           st.kind == StepKind::RulebookInverse;
+  };
+  auto fail = [](const Step& st, int rc) {
+    SCN_LOGE("forward failed at step %s", st.label.c_str());
+    return rc;
+  };
   if (dual) {
+    int aux_seq = 0, waited_seq = 0;
     e->rb_seq.assign(e->rulebooks.size(), 0);
     e->coord_rb.assign(e->coords.size(), -1);
+    e->map_built.assign(e->steps.size(), 0);
+    // pass 1: the input count (which also clears what the coordinate kernels build into), then the
+    // coordinate steps
+    for (size_t si = 0; si < e->steps.size(); ++si) {
+      Step& st = e->steps[si];
+      if (st.kind == StepKind::InputCount) {
+        int rc = run_step(*e, st, stream);
+        if (rc) return fail(st, rc);
+        SCN_HIP(hipEventRecord(e->ev_fork, stream));
+        SCN_HIP(hipStreamWaitEvent(e->aux, e->ev_fork, 0));
+      } else if (is_coord_step(st)) {
+        int rc = run_step(*e, st, e->aux);
+        if (rc) return fail(st, rc);
+        if (st.kind != StepKind::HashBuild) {
+          SCN_HIP(hipEventRecord(e->rb_ready[st.rulebook], e->aux));
+          e->rb_seq[st.rulebook] = ++aux_seq;
+          if (st.kind == StepKind::RulebookSparse) e->coord_rb[e->rulebooks[st.rulebook]->coord_out] = st.rulebook;
+        }
+      } else if (st.kind == StepKind::Dense && si < e->dense_maps.size() && e->dense_maps[si].p &&
+                 e->dense_precleared[si] == 2) {
+        const CoordSet& cs = e->coords[e->tensors[st.t_in].coord];
+        int rc = scatter_dense_build_map(cs.idx, cs.n_bound, cs.n_dev, st.dense_shape, st.has_perm ? st.perm : nullptr,
+                                         e->dense_maps[si].as<int32_t>(), true, e->aux);
+        if (rc) return fail(st, rc);
+        e->map_built[si] = 1;
+      }
+    }
+    SCN_HIP(hipEventRecord(e->ev_join, e->aux));
+    // pass 2: the feature kernels
+    for (size_t si = 0; si < e->steps.size(); ++si) {
+      Step& st = e->steps[si];
+      if (st.kind == StepKind::InputCount || is_coord_step(st)) continue;
+      // rulebook this step depends on: its own (convolutions) or the one that produced its rows
+      int rb = -1;
+      if (st.kind == StepKind::Conv) {
+        rb = st.rulebook;
+      } else if (st.t_in >= 0 && st.t_in < (int)e->tensors.size()) {
+        const int c = e->tensors[st.t_in].coord;
+        if (c >= 0 && c < (int)e->coord_rb.size()) rb = e->coord_rb[c];
+      }
+      if (e->map_built[si] && waited_seq <= aux_seq) {
+        SCN_HIP(hipStreamWaitEvent(stream, e->ev_join, 0));  // row maps come after every rulebook
+        waited_seq = aux_seq + 1;
+      } else if (rb >= 0 && e->rb_seq[rb] > waited_seq) {
+        SCN_HIP(hipStreamWaitEvent(stream, e->rb_ready[rb], 0));
+        waited_seq = e->rb_seq[rb];
+      }
+      e->dense_map_built = e->map_built[si] != 0;
+      int rc = run_step(*e, st, stream);
+      e->dense_map_built = false;
+      if (rc) return fail(st, rc);
+    }
+    SCN_HIP(hipStreamWaitEvent(stream, e->ev_join, 0));
+    return SCN_OK;
   }
   for (auto& st : e->steps) {
     if (e->profiling) {
@@ -1673,61 +1736,9 @@ int scn_engine_forward(scn_engine* e, void* stream_) {
       }
       SCN_HIP(hipEventRecord(st.ev0, stream));
     }
-    const bool coord_step =
-        st.kind == StepKind::HashBuild || st.kind == StepKind::RulebookSubm || st.kind == StepKind::RulebookSparse ||
-        st.kind == StepKind::RulebookInverse;
-    hipStream_t run_on = stream;
-    if (dual && coord_step) {
-      run_on = e->aux;
-    } else if (dual && st.kind != StepKind::InputCount) {
-      // rulebook this step depends on: its own (convolutions) or the one that produced its rows
-      int rb = -1;
-      if (st.kind == StepKind::Conv) {
-        rb = st.rulebook;
-      } else if (st.t_in >= 0 && st.t_in < (int)e->tensors.size()) {
-        const int c = e->tensors[st.t_in].coord;
-        if (c >= 0 && c < (int)e->coord_rb.size()) rb = e->coord_rb[c];
-      }
-      if (rb >= 0 && e->rb_seq[rb] > waited_seq) {
-        SCN_HIP(hipStreamWaitEvent(stream, e->rb_ready[rb], 0));
-        waited_seq = e->rb_seq[rb];
-      }
-    }
-    if (dual && st.kind == StepKind::Dense) {
-      // The row map needs only the coordinates, which the auxiliary stream has produced (or which came
-      // with the input): build it there, ahead of the convolutions the main stream is still running.
-      const size_t si = (size_t)(&st - e->steps.data());
-      if (si < e->dense_maps.size() && e->dense_maps[si].p && e->dense_precleared[si] == 2) {
-        const CoordSet& cs = e->coords[e->tensors[st.t_in].coord];
-        int rc = scatter_dense_build_map(cs.idx, cs.n_bound, cs.n_dev, st.dense_shape, st.has_perm ? st.perm : nullptr,
-                                         e->dense_maps[si].as<int32_t>(), true, e->aux);
-        if (rc) return rc;
-        SCN_HIP(hipEventRecord(e->ev_map, e->aux));
-        SCN_HIP(hipStreamWaitEvent(stream, e->ev_map, 0));
-        e->dense_map_built = true;
-      }
-    }
-    int rc = run_step(*e, st, run_on);
-    e->dense_map_built = false;
-    if (rc) {
-      SCN_LOGE("forward failed at step %s", st.label.c_str());
-      return rc;
-    }
-    if (dual && st.kind == StepKind::InputCount) {
-      SCN_HIP(hipEventRecord(e->ev_fork, stream));
-      SCN_HIP(hipStreamWaitEvent(e->aux, e->ev_fork, 0));
-    }
-    if (dual && (st.kind == StepKind::RulebookSubm || st.kind == StepKind::RulebookSparse ||
-                 st.kind == StepKind::RulebookInverse)) {
-      SCN_HIP(hipEventRecord(e->rb_ready[st.rulebook], e->aux));
-      e->rb_seq[st.rulebook] = ++aux_seq;
-      if (st.kind == StepKind::RulebookSparse) e->coord_rb[e->rulebooks[st.rulebook]->coord_out] = st.rulebook;
-    }
+    int rc = run_step(*e, st, stream);
+    if (rc) return fail(st, rc);
     if (e->profiling) SCN_HIP(hipEventRecord(st.ev1, stream));
-  }
-  if (dual) {
-    SCN_HIP(hipEventRecord(e->ev_join, e->aux));
-    SCN_HIP(hipStreamWaitEvent(stream, e->ev_join, 0));
   }
   if (e->profiling) {
     SCN_HIP(hipStreamSynchronize(stream));
