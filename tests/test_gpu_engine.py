@@ -540,3 +540,25 @@ def test_implicit_calibration_collect_amax_and_ranges(cp_models, centerpoint_inp
     assert r.returncode == 0, r.stdout
     out = tensor.load(prefix + ".0.tensor")
     assert np.array_equal(out.view(np.uint16), want.view(np.uint16))
+
+
+def test_inverted_graph_on_device_gives_the_same_bev(bevfusion_input):
+    """xyz -> zyx inversion of an all-int8 BEVFusion-shaped model (`CUDA-BEVFusion/qat/lean/exptool.py:332-343`):
+    integer arithmetic end to end, so the dense output must not change by one bit, on the device as in the oracle."""
+    from lidar_ai_solution_amd import export
+    feats, idx = bevfusion_input
+    note("all-int8 BEVFusion-shaped backbone, xyz and inverted (zyx) on the same frame")
+    g16, _ = graphs.bevfusion_scn(seed=6)
+    amax = _oracle_calibration(g16, feats, idx, GRID_XYZ)
+    g8, tags8 = graphs.bevfusion_scn(seed=6)
+    graphs.apply_int8_plan(g8, tags8, amax, "all-int8")
+    want = O.run_graph(g8, feats, idx, GRID_XYZ, "int8")[g8.outputs[0]]
+    eng = Engine.from_graph(g8, "int8")
+    _run_engine(eng, feats, idx, GRID_XYZ)
+    got = eng.output(0).torch().cpu().numpy()
+    assert np.count_nonzero(want) > 10000 and np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    gi = export.invert_graph(g8)
+    eng_i = Engine.from_graph(gi, "int8")
+    _run_engine(eng_i, feats, export.invert_indices(idx), GRID_XYZ[::-1])
+    got_i = eng_i.output(0).torch().cpu().numpy()
+    assert got_i.shape == want.shape and np.array_equal(got_i.view(np.uint16), want.view(np.uint16))
