@@ -160,6 +160,10 @@ int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, cons
   a.res_dtype = io.res_dtype;
   a.res_scale = s_of(io.res_dynamic_range);
   a.res_ld = io.res_ld;
+  {
+    const size_t rsz = io.res_dtype == SCN_DTYPE_INT8 ? 1 : 2;
+    a.res_vec16 = (io.res_dev && ((size_t)io.res_ld * rsz) % 16 == 0 && ((uintptr_t)io.res_dev & 15) == 0) ? 1 : 0;
+  }
   a.mid_dtype = io.mid_dtype;
   a.mid_s = s_of(io.mid_dynamic_range);
   a.mid_r = r_of(io.mid_dynamic_range);

@@ -29,6 +29,7 @@ struct ConvArgs {
   int res_dtype;
   float res_scale;          // amax_res / 127
   uint32_t res_ld;
+  int res_vec16;            // residual rows are 16-byte aligned and a multiple of 16 bytes
   int mid_dtype;
   float mid_s, mid_r;       // amax_mid / 127, 127 / amax_mid
   float a_rq_s, a_rq_r;     // re-quantisation of an fp16 operand by an int8 Add (0 = none)

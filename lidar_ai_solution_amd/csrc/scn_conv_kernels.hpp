@@ -3,6 +3,8 @@
 // compile side by side.
 #pragma once
 
+#include <type_traits>
+
 #include "scn_conv_args.hpp"
 #include "scn_device.hpp"
 
@@ -64,25 +66,36 @@ __device__ __forceinline__ bool xcd_tile(uint32_t n, uint32_t rows_per_block, ui
 // Fused epilogue of 4 consecutive channels of one row: bias, requantisation scale, ReLU, residual add
 // (with the mid-quantisation the un-fused graph would have applied), second ReLU.  Also dumps the raw
 // accumulators when asked to.  y[] receives the values to store.
-template <int EL>
+//   b4   bias of the 4 channels
+//   sc4  int8: s_x * s_w[c] of the 4 channels (one fp32 rounding); unused for fp16
+//   resp the 4 residual values of this row (a.res_dtype), in global memory or staged in LDS; unused
+//        without a residual
+//   MODE 0: every switch is read from the arguments.  The others fix the combinations the backbones use
+//        at compile time, because 16 unrolled pieces of the general code are ~11,000 instructions, more
+//        than the instruction cache holds, and the epilogue then runs at the speed of its fetches:
+//        1 / 2: no accumulator dump, no residual, int8 / fp16 output
+//        3 / 4: no dump, residual and un-fused intermediate both int8 / both fp16 (same type as the output)
+template <int EL, int MODE = 0>
 __device__ __forceinline__ void epilogue_values(const ConvArgs& a, uint32_t row, int co,
-                                                const typename Mma<EL>::Acc& acc, float y[4]) {
-  const float4 bs = *reinterpret_cast<const float4*>(a.bias + co);
-  const float b4[4] = {bs.x, bs.y, bs.z, bs.w};
+                                                const typename Mma<EL>::Acc& acc, const float4 b4v, const float4 sc4v,
+                                                const void* resp, float y[4]) {
+  const bool dump = MODE == 0 && a.acc != nullptr;
+  const bool has_res = MODE == 0 ? a.res != nullptr : MODE >= 3;
+  const bool res8 = MODE == 0 ? a.res_dtype == SCN_DTYPE_INT8 : MODE == 3;
+  const bool mid8 = MODE == 0 ? a.mid_dtype == SCN_DTYPE_INT8 : MODE == 3;
+  const float b4[4] = {b4v.x, b4v.y, b4v.z, b4v.w};
   if (EL == 0) {
-    const float4 ws = *reinterpret_cast<const float4*>(a.wscale + co);
-    const float w4[4] = {ws.x, ws.y, ws.z, ws.w};
+    const float sc4[4] = {sc4v.x, sc4v.y, sc4v.z, sc4v.w};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const float sc = a.x_scale * w4[j];         // s_x * s_w[c], one fp32 rounding
-      const float m = (float)acc[j] * sc;          // fp32 multiply
+      const float m = (float)acc[j] * sc4[j];      // fp32 multiply
       y[j] = m + b4[j];                            // fp32 add (the library is built with -ffp-contract=off)
     }
   } else {
 #pragma unroll
     for (int j = 0; j < 4; ++j) y[j] = (float)acc[j] + b4[j];
   }
-  if (a.acc) {
+  if (dump) {
     if (EL == 0)
       *reinterpret_cast<v4i*>((int32_t*)a.acc + (size_t)row * a.cout + co) = __builtin_bit_cast(v4i, acc);
     else
@@ -92,17 +105,17 @@ __device__ __forceinline__ void epilogue_values(const ConvArgs& a, uint32_t row,
 #pragma unroll
     for (int j = 0; j < 4; ++j) y[j] = y[j] > 0.f ? y[j] : 0.f;
   }
-  if (a.res) {
+  if (has_res) {
     // value of the un-fused conv output as its consumer (the Add) would have read it
     float rv[4];
-    if (a.res_dtype == SCN_DTYPE_INT8) {
-      const char4 r = *reinterpret_cast<const char4*>(a.res + (size_t)row * a.res_ld + co);
+    if (res8) {
+      const char4 r = *reinterpret_cast<const char4*>(resp);
       rv[0] = (float)r.x * a.res_scale;
       rv[1] = (float)r.y * a.res_scale;
       rv[2] = (float)r.z * a.res_scale;
       rv[3] = (float)r.w * a.res_scale;
     } else {
-      const _Float16* r = reinterpret_cast<const _Float16*>(a.res) + (size_t)row * a.res_ld + co;
+      const _Float16* r = reinterpret_cast<const _Float16*>(resp);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         rv[j] = (float)r[j];
@@ -112,7 +125,7 @@ __device__ __forceinline__ void epilogue_values(const ConvArgs& a, uint32_t row,
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       float v;
-      if (a.mid_dtype == SCN_DTYPE_INT8) {
+      if (mid8) {
         v = quant_f(y[j], a.mid_r) * a.mid_s;
       } else {
         v = half_round(y[j]);
@@ -123,6 +136,11 @@ __device__ __forceinline__ void epilogue_values(const ConvArgs& a, uint32_t row,
       y[j] = v;
     }
   }
+}
+
+// Address of the 4 residual values of (row, co) in global memory.
+__device__ __forceinline__ const void* residual_ptr(const ConvArgs& a, uint32_t row, int co) {
+  return a.res + ((size_t)row * a.res_ld + co) * (a.res_dtype == SCN_DTYPE_INT8 ? 1 : 2);
 }
 
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
@@ -140,15 +158,73 @@ __device__ __forceinline__ v4h pack_fp16(const float y[4]) {
   return v4h{(_Float16)y[0], (_Float16)y[1], (_Float16)y[2], (_Float16)y[3]};
 }
 
+// One rounded, clamped value -> byte BYTE of the packed word (the conversion writes the byte itself,
+// so no shifts and masks are needed to pack four of them).
+#define SCN_CVT_BYTE(BYTE, PACKED, Q) \
+  asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_" #BYTE " dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(PACKED) : "v"(Q))
+
+// The int8-output modes 1 and 3 of epilogue_values() without a branch: the same operations in the same
+// order, except that a ReLU directly in front of a quantiser is the quantiser's lower clamp (0 instead
+// of -127: rounding a negative product gives a value <= -0, which clamps to 0 either way).
+//   lo1  lower clamp of the first quantiser after the convolution's own ReLU switch (a.relu ? 0 : -127):
+//        the output quantiser (mode 1) or the un-fused intermediate's (mode 3)
+//   lo2  mode 3: lower clamp of the output quantiser (a.relu2 ? 0 : -127)
+//   r4   mode 3: the 4 residual bytes
+template <int EL, int MODE>
+__device__ __forceinline__ uint32_t epilogue_pack8(const ConvArgs& a, const typename Mma<EL>::Acc& acc, const float4 b4v,
+                                                   const float4 sc4v, float lo1, float lo2, uint32_t r4) {
+  static_assert(MODE == 1 || MODE == 3, "int8-output modes only");
+  const float b4[4] = {b4v.x, b4v.y, b4v.z, b4v.w};
+  const float sc4[4] = {sc4v.x, sc4v.y, sc4v.z, sc4v.w};
+  float q[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float y;
+    if (EL == 0) {
+      const float m = (float)acc[j] * sc4[j];
+      y = m + b4[j];
+    } else {
+      y = (float)acc[j] + b4[j];
+    }
+    if (MODE == 1) {
+      q[j] = __builtin_amdgcn_fmed3f(rintf(y * a.out_r), lo1, 127.f);
+    } else {
+      const float mid = __builtin_amdgcn_fmed3f(rintf(y * a.mid_r), lo1, 127.f) * a.mid_s;
+      const float rv = (float)(int)(signed char)(r4 >> (8 * j)) * a.res_scale;
+      const float v = mid + rv;
+      q[j] = __builtin_amdgcn_fmed3f(rintf(v * a.out_r), lo2, 127.f);
+    }
+  }
+  uint32_t packed = 0;
+  SCN_CVT_BYTE(0, packed, q[0]);
+  SCN_CVT_BYTE(1, packed, q[1]);
+  SCN_CVT_BYTE(2, packed, q[2]);
+  SCN_CVT_BYTE(3, packed, q[3]);
+  return packed;
+}
+#undef SCN_CVT_BYTE
+
 // Stores 4 consecutive channels of one row after the fused epilogue.
 template <int EL>
-__device__ __forceinline__ void epilogue_store(const ConvArgs& a, uint32_t row, int co, const typename Mma<EL>::Acc& acc) {
+__device__ __forceinline__ void epilogue_store(const ConvArgs& a, uint32_t row, int co, const typename Mma<EL>::Acc& acc,
+                                               const float4 b4, const float4 sc4) {
   float y[4];
-  epilogue_values<EL>(a, row, co, acc, y);
+  epilogue_values<EL>(a, row, co, acc, b4, sc4, a.res ? residual_ptr(a, row, co) : nullptr, y);
   if (a.out_dtype == SCN_DTYPE_INT8)
     *reinterpret_cast<char4*>(a.out + (size_t)row * a.out_ld + co) = pack_int8(a, y);
   else
     *reinterpret_cast<v4h*>(reinterpret_cast<_Float16*>(a.out) + (size_t)row * a.out_ld + co) = pack_fp16(y);
+}
+
+// Bias and (int8) full requantisation scale of 4 channels from global memory.
+template <int EL>
+__device__ __forceinline__ void epilogue_consts(const ConvArgs& a, int co, float4* b4, float4* sc4) {
+  *b4 = *reinterpret_cast<const float4*>(a.bias + co);
+  *sc4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (EL == 0) {
+    const float4 ws = *reinterpret_cast<const float4*>(a.wscale + co);
+    *sc4 = make_float4(a.x_scale * ws.x, a.x_scale * ws.y, a.x_scale * ws.z, a.x_scale * ws.w);  // s_x * s_w[c]
+  }
 }
 
 // Row-split kernel: each wave owns 16*NT output rows and all MT*16 output channels; both operands
@@ -232,7 +308,11 @@ __global__ __launch_bounds__(256) void k_conv_rows(const ConvArgs a) {
   for (int u = 0; u < NT; ++u) {
     if (rows[u] >= n) continue;
 #pragma unroll
-    for (int t = 0; t < MT; ++t) epilogue_store<EL>(a, rows[u], t * 16 + lg * 4, acc[t][u]);
+    for (int t = 0; t < MT; ++t) {
+      float4 b4, sc4;
+      epilogue_consts<EL>(a, t * 16 + lg * 4, &b4, &sc4);
+      epilogue_store<EL>(a, rows[u], t * 16 + lg * 4, acc[t][u], b4, sc4);
+    }
   }
 }
 
@@ -503,12 +583,20 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
 #undef SCN_SLAB
 #undef SCN_INDEX
 #undef SCN_GATHER
-  // Epilogue.  Each lane holds 4-channel pieces of one row; writing them directly would touch every
-  // 128-byte line of the tile 16 times.  The pieces go through the wave's LDS stage instead (same XOR
-  // placement as the gathers) and leave as 16 bytes per lane, 8 lanes per row.
+  // Epilogue.  Nothing in it may wait for global memory once per 4-channel piece (16 pieces per lane
+  // for 128 channels, each a cache round trip): the per-channel constants are staged in LDS once per
+  // workgroup, in the weight slab's space, and a residual tile is staged per wave like the output.
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stage still receives the gathers issued past the end
-  const uint32_t row = row0 + ln;
+  asm volatile("s_barrier" ::: "memory");           // ... and the slab buffers every wave's re-loads of the last slab
+  float* ep = reinterpret_cast<float*>(&lds[0][0]);  // [0, 128): bias, [128, 256): s_x * s_w[c]
   const int cout_pad = (a.cout + 15) & ~15;
+  if (tid < MT * 32) {
+    const bool okc = tid < cout_pad;
+    ep[tid] = okc ? a.bias[tid] : 0.f;
+    if (EL == 0) ep[128 + tid] = okc ? a.x_scale * a.wscale[tid] : 0.f;
+  }
+  __syncthreads();
+  const uint32_t row = row0 + ln;
   if (!a.out_vec16) {
     if (row >= n) return;
 #pragma unroll
@@ -518,50 +606,97 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
         const int co = t * 32 + g * 8 + lh * 4;
         if (co >= cout_pad) continue;
         const Acc4 piece = {acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
-        epilogue_store<EL>(a, row, co, piece);
+        epilogue_store<EL>(a, row, co, piece, *reinterpret_cast<const float4*>(ep + co),
+                           *reinterpret_cast<const float4*>(ep + 128 + co));
       }
     return;
   }
+  // Each lane holds 4-channel pieces of one row; writing them directly would touch every 128-byte line
+  // of the tile 16 times.  The pieces go through the wave's LDS stage instead (same XOR placement as the
+  // gathers) and leave as 16 bytes per lane, 8 lanes per row.  A residual of the output's element size
+  // comes in the same way first: each piece finds its 4 residual values in the slot it then overwrites.
   char* stage = reinterpret_cast<char*>(&ring[wave][0]);
   const bool out8 = a.out_dtype == SCN_DTYPE_INT8;
+  const bool res_staged = a.res && a.res_vec16 && a.res_dtype == a.out_dtype;
   constexpr int PASSES = MT >= 4 ? 2 : 1;          // fp16 rows of 128 channels take two 128-byte passes
   constexpr int TPP = MT >= 4 ? 2 : MT;            // 32-channel tiles per fp16 pass
+  auto run = [&](auto mode_c) {
+    constexpr int MODE = decltype(mode_c)::value;
+    const bool o8 = MODE == 0 ? out8 : (MODE == 1 || MODE == 3);
+    const bool staged = MODE == 0 ? res_staged : MODE >= 3;
+    const float lo1 = a.relu ? 0.f : -127.f, lo2 = a.relu2 ? 0.f : -127.f;
 #pragma unroll
-  for (int p = 0; p < PASSES; ++p) {
-    if (out8 && p > 0) break;
-    const int t_lo = out8 ? 0 : p * TPP, t_hi = out8 ? MT : p * TPP + TPP;
-    const int c0 = t_lo * 32;                      // first channel of the pass
+    for (int p = 0; p < PASSES; ++p) {
+      if (o8 && p > 0) break;
+      const int t_lo = o8 ? 0 : p * TPP, t_hi = o8 ? MT : p * TPP + TPP;
+      const int c0 = t_lo * 32;                      // first channel of the pass
+      const int osz = o8 ? 1 : 2;
+      const int valid = (cout_pad - c0) * osz;       // bytes of the pass row that exist
+      if (staged) {
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      if (t < t_lo || t >= t_hi) continue;
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int co = t * 32 + g * 8 + lh * 4;
-        if (co >= cout_pad || row >= n) continue;
-        const Acc4 piece = {acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
-        float y[4];
-        epilogue_values<EL>(a, row, co, piece, y);
-        const int off = (co - c0) * (out8 ? 1 : 2);  // byte offset inside the 128-byte pass row
-        char* dst = stage + ln * 128 + (((off >> 4) ^ (ln & 7)) << 4) + (off & 15);
-        if (out8)
-          *reinterpret_cast<char4*>(dst) = pack_int8(a, y);
-        else
-          *reinterpret_cast<v4h*>(dst) = pack_fp16(y);
+        for (int j = 0; j < 4; ++j) {
+          const int r = (lane >> 3) + 8 * j, c = lane & 7;
+          const uint32_t grow = row0 + r;
+          v4i v = {0, 0, 0, 0};
+          if (grow < n && c * 16 < valid)
+            v = *reinterpret_cast<const v4i*>(a.res + ((size_t)grow * a.res_ld + c0) * osz + c * 16);
+          *reinterpret_cast<v4i*>(stage + r * 128 + ((c ^ (r & 7)) << 4)) = v;
+        }
       }
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    const int osz = out8 ? 1 : 2;
-    const int valid = (cout_pad - c0) * osz;       // bytes of the pass row that exist
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int r = (lane >> 3) + 8 * j, c = lane & 7;
-      const uint32_t grow = row0 + r;
-      if (grow < n && c * 16 < valid) {
-        const v4i v = *reinterpret_cast<const v4i*>(stage + r * 128 + ((c ^ (r & 7)) << 4));
-        *reinterpret_cast<v4i*>(a.out + ((size_t)grow * a.out_ld + c0) * osz + c * 16) = v;
+      for (int t = 0; t < MT; ++t) {
+        if (t < t_lo || t >= t_hi) continue;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int co = t * 32 + g * 8 + lh * 4;
+          // (the specialised modes touch nothing but LDS here: lanes without a row or channel run along)
+          if (MODE == 0 && (co >= cout_pad || row >= n)) continue;
+          const Acc4 piece = {acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
+          const int off = (co - c0) * osz;           // byte offset inside the 128-byte pass row
+          char* dst = stage + ln * 128 + (((off >> 4) ^ (ln & 7)) << 4) + (off & 15);
+          if constexpr (MODE == 1 || MODE == 3) {
+            const uint32_t r4 = MODE == 3 ? *reinterpret_cast<const uint32_t*>(dst) : 0u;
+            *reinterpret_cast<uint32_t*>(dst) =
+                epilogue_pack8<EL, MODE>(a, piece, *reinterpret_cast<const float4*>(ep + co),
+                                         *reinterpret_cast<const float4*>(ep + 128 + co), lo1, lo2, r4);
+            continue;
+          }
+          float y[4];
+          epilogue_values<EL, MODE>(a, row, co, piece, *reinterpret_cast<const float4*>(ep + co),
+                              *reinterpret_cast<const float4*>(ep + 128 + co),
+                              staged ? (const void*)dst : (a.res ? residual_ptr(a, row, co) : nullptr), y);
+          if (o8)
+            *reinterpret_cast<char4*>(dst) = pack_int8(a, y);
+          else
+            *reinterpret_cast<v4h*>(dst) = pack_fp16(y);
+        }
       }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int r = (lane >> 3) + 8 * j, c = lane & 7;
+        const uint32_t grow = row0 + r;
+        if (grow < n && c * 16 < valid) {
+          const v4i v = *reinterpret_cast<const v4i*>(stage + r * 128 + ((c ^ (r & 7)) << 4));
+          *reinterpret_cast<v4i*>(a.out + ((size_t)grow * a.out_ld + c0) * osz + c * 16) = v;
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  };
+  int mode = 0;
+  if (!a.acc) {
+    if (!a.res)
+      mode = out8 ? 1 : 2;
+    else if (res_staged && a.mid_dtype == a.out_dtype)
+      mode = out8 ? 3 : 4;
+  }
+  switch (mode) {
+    case 1: run(std::integral_constant<int, 1>{}); break;
+    case 2: run(std::integral_constant<int, 2>{}); break;
+    case 3: run(std::integral_constant<int, 3>{}); break;
+    case 4: run(std::integral_constant<int, 4>{}); break;
+    default: run(std::integral_constant<int, 0>{}); break;
   }
 }
 
