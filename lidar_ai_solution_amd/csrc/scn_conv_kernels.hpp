@@ -204,6 +204,32 @@ __device__ __forceinline__ uint32_t epilogue_pack8(const ConvArgs& a, const type
 }
 #undef SCN_CVT_BYTE
 
+// The fp16-output modes 2 and 4 of epilogue_values() without a branch (mode 4 is only chosen when neither
+// operand of the fused Add is re-quantised).  lo1 / lo2: 0 where the ReLU switch is on, -inf where it is off.
+template <int EL, int MODE>
+__device__ __forceinline__ v4h epilogue_pack16(const typename Mma<EL>::Acc& acc, const float4 b4v, const float4 sc4v,
+                                               float lo1, float lo2, v4h r4) {
+  static_assert(MODE == 2 || MODE == 4, "fp16-output modes only");
+  const float b4[4] = {b4v.x, b4v.y, b4v.z, b4v.w};
+  const float sc4[4] = {sc4v.x, sc4v.y, sc4v.z, sc4v.w};
+  float y[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (EL == 0) {
+      const float m = (float)acc[j] * sc4[j];
+      y[j] = m + b4[j];
+    } else {
+      y[j] = (float)acc[j] + b4[j];
+    }
+    y[j] = y[j] > lo1 ? y[j] : lo1;
+    if (MODE == 4) {
+      const float v = half_round(y[j]) + (float)r4[j];
+      y[j] = v > lo2 ? v : lo2;
+    }
+  }
+  return pack_fp16(y);
+}
+
 // Stores 4 consecutive channels of one row after the fused epilogue.
 template <int EL>
 __device__ __forceinline__ void epilogue_store(const ConvArgs& a, uint32_t row, int co, const typename Mma<EL>::Acc& acc,
@@ -587,15 +613,42 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
   // for 128 channels, each a cache round trip): the per-channel constants are staged in LDS once per
   // workgroup, in the weight slab's space, and a residual tile is staged per wave like the output.
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stage still receives the gathers issued past the end
-  asm volatile("s_barrier" ::: "memory");           // ... and the slab buffers every wave's re-loads of the last slab
-  float* ep = reinterpret_cast<float*>(&lds[0][0]);  // [0, 128): bias, [128, 256): s_x * s_w[c]
   const int cout_pad = (a.cout + 15) & ~15;
-  if (tid < MT * 32) {
-    const bool okc = tid < cout_pad;
-    ep[tid] = okc ? a.bias[tid] : 0.f;
-    if (EL == 0) ep[128 + tid] = okc ? a.x_scale * a.wscale[tid] : 0.f;
+  float* ep = reinterpret_cast<float*>(&lds[0][0]);  // [0, 128): bias, [128, 256): s_x * s_w[c]
+  float4 cb[MT == 1 ? 4 : 1], cs[MT == 1 ? 4 : 1];
+  if constexpr (MT == 1) {
+    // 32 output channels are 4 pieces per lane: their constants fit registers and arrive in one round
+    // trip, without the two barriers below (these layers are short; a barrier is a visible part of them)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int co = g * 8 + lh * 4;
+      const int cc = co < cout_pad ? co : 0;
+      cb[g] = *reinterpret_cast<const float4*>(a.bias + cc);
+      cs[g] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (EL == 0) {
+        const float4 ws = *reinterpret_cast<const float4*>(a.wscale + cc);
+        cs[g] = make_float4(a.x_scale * ws.x, a.x_scale * ws.y, a.x_scale * ws.z, a.x_scale * ws.w);
+      }
+    }
+  } else {
+    asm volatile("s_barrier" ::: "memory");         // the slab buffers received every wave's re-loads of the last slab
+    if (tid < MT * 32) {
+      const bool okc = tid < cout_pad;
+      ep[tid] = okc ? a.bias[tid] : 0.f;
+      if (EL == 0) ep[128 + tid] = okc ? a.x_scale * a.wscale[tid] : 0.f;
+    }
+    __syncthreads();
   }
-  __syncthreads();
+  // constants of piece g of tile t (channels co .. co + 3)
+  auto consts = [&](int g, int co, float4* b4, float4* sc4) {
+    if constexpr (MT == 1) {
+      *b4 = cb[g];
+      *sc4 = cs[g];
+    } else {
+      *b4 = *reinterpret_cast<const float4*>(ep + co);
+      *sc4 = *reinterpret_cast<const float4*>(ep + 128 + co);
+    }
+  };
   const uint32_t row = row0 + ln;
   if (!a.out_vec16) {
     if (row >= n) return;
@@ -606,8 +659,9 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
         const int co = t * 32 + g * 8 + lh * 4;
         if (co >= cout_pad) continue;
         const Acc4 piece = {acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
-        epilogue_store<EL>(a, row, co, piece, *reinterpret_cast<const float4*>(ep + co),
-                           *reinterpret_cast<const float4*>(ep + 128 + co));
+        float4 b4, sc4;
+        consts(g, co, &b4, &sc4);
+        epilogue_store<EL>(a, row, co, piece, b4, sc4);
       }
     return;
   }
@@ -617,14 +671,16 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
   // comes in the same way first: each piece finds its 4 residual values in the slot it then overwrites.
   char* stage = reinterpret_cast<char*>(&ring[wave][0]);
   const bool out8 = a.out_dtype == SCN_DTYPE_INT8;
-  const bool res_staged = a.res && a.res_vec16 && a.res_dtype == a.out_dtype;
+  // (16-channel rows are one 16-byte chunk: staging them costs more than the two 4-byte reads it replaces)
+  const bool res_staged = a.res && a.res_vec16 && a.res_dtype == a.out_dtype && cout_pad >= 32;
   constexpr int PASSES = MT >= 4 ? 2 : 1;          // fp16 rows of 128 channels take two 128-byte passes
   constexpr int TPP = MT >= 4 ? 2 : MT;            // 32-channel tiles per fp16 pass
   auto run = [&](auto mode_c) {
     constexpr int MODE = decltype(mode_c)::value;
     const bool o8 = MODE == 0 ? out8 : (MODE == 1 || MODE == 3);
     const bool staged = MODE == 0 ? res_staged : MODE >= 3;
-    const float lo1 = a.relu ? 0.f : -127.f, lo2 = a.relu2 ? 0.f : -127.f;
+    const float lo1 = a.relu ? 0.f : -127.f, lo2 = a.relu2 ? 0.f : -127.f;          // int8 clamps
+    const float lo1h = a.relu ? 0.f : -__builtin_inff(), lo2h = a.relu2 ? 0.f : -__builtin_inff();
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       if (o8 && p > 0) break;
@@ -651,19 +707,24 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
           const int co = t * 32 + g * 8 + lh * 4;
           // (the specialised modes touch nothing but LDS here: lanes without a row or channel run along)
           if (MODE == 0 && (co >= cout_pad || row >= n)) continue;
+          if (MT == 1 && t * 32 + g * 8 >= cout_pad) continue;  // narrow layers: skip the padding pieces (uniform)
           const Acc4 piece = {acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
           const int off = (co - c0) * osz;           // byte offset inside the 128-byte pass row
           char* dst = stage + ln * 128 + (((off >> 4) ^ (ln & 7)) << 4) + (off & 15);
+          float4 b4, sc4;
+          consts(g, co, &b4, &sc4);
           if constexpr (MODE == 1 || MODE == 3) {
             const uint32_t r4 = MODE == 3 ? *reinterpret_cast<const uint32_t*>(dst) : 0u;
-            *reinterpret_cast<uint32_t*>(dst) =
-                epilogue_pack8<EL, MODE>(a, piece, *reinterpret_cast<const float4*>(ep + co),
-                                         *reinterpret_cast<const float4*>(ep + 128 + co), lo1, lo2, r4);
+            *reinterpret_cast<uint32_t*>(dst) = epilogue_pack8<EL, MODE>(a, piece, b4, sc4, lo1, lo2, r4);
+            continue;
+          }
+          if constexpr (MODE == 2 || MODE == 4) {
+            const v4h r4 = MODE == 4 ? *reinterpret_cast<const v4h*>(dst) : v4h{0, 0, 0, 0};
+            *reinterpret_cast<v4h*>(dst) = epilogue_pack16<EL, MODE>(piece, b4, sc4, lo1h, lo2h, r4);
             continue;
           }
           float y[4];
-          epilogue_values<EL, MODE>(a, row, co, piece, *reinterpret_cast<const float4*>(ep + co),
-                              *reinterpret_cast<const float4*>(ep + 128 + co),
+          epilogue_values<EL, MODE>(a, row, co, piece, b4, sc4,
                               staged ? (const void*)dst : (a.res ? residual_ptr(a, row, co) : nullptr), y);
           if (o8)
             *reinterpret_cast<char4*>(dst) = pack_int8(a, y);
@@ -688,7 +749,7 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
   if (!a.acc) {
     if (!a.res)
       mode = out8 ? 1 : 2;
-    else if (res_staged && a.mid_dtype == a.out_dtype)
+    else if (res_staged && a.mid_dtype == a.out_dtype && (out8 || (a.a_rq_r <= 0.f && a.b_rq_r <= 0.f)))
       mode = out8 ? 3 : 4;
   }
   switch (mode) {
