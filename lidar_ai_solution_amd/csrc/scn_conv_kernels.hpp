@@ -539,12 +539,13 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
     SCN_INDEX(3);
   }
   SCN_SLAB(0);
-  SCN_WAIT_VM(0);
+  SCN_WAIT_VM((DEPTH - 1) * IDXI + WPT);  // I(0), the oldest, has landed
   {
     int32_t gi[4];
     SCN_READ_INDEX(0, gi);
     SCN_GATHER(0, gi);
   }
+  SCN_WAIT_VM(4);  // ... and this wave's part of S(0) (younger: G(0))
   asm volatile("s_barrier" ::: "memory");
 
   for (int it = 0; it < iters; ++it) {
