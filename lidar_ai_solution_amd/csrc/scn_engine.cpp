@@ -1675,15 +1675,32 @@ int scn_engine_forward(scn_engine* e, void* stream_) {
     e->coord_rb.assign(e->coords.size(), -1);
     e->map_built.assign(e->steps.size(), 0);
     // pass 1: the input count (which also clears what the coordinate kernels build into), then the
-    // coordinate steps
+    // coordinate steps.  What the first convolution needs (the input hash and its rulebook) stays on the
+    // caller's stream: a dependency across streams costs ~12 us from the event to the dependent kernel's
+    // start when the waiting stream is idle, and the first convolution would pay that twice (fork and
+    // wait).  The auxiliary stream starts as soon as the coordinates and look-ups it reads exist.
+    size_t first_conv = e->steps.size();
+    for (size_t si = 0; si < e->steps.size(); ++si)
+      if (e->steps[si].kind == StepKind::Conv) {
+        first_conv = si;
+        break;
+      }
+    bool aux_started = false;
     for (size_t si = 0; si < e->steps.size(); ++si) {
       Step& st = e->steps[si];
       if (st.kind == StepKind::InputCount) {
         int rc = run_step(*e, st, stream);
         if (rc) return fail(st, rc);
         SCN_HIP(hipEventRecord(e->ev_fork, stream));
-        SCN_HIP(hipStreamWaitEvent(e->aux, e->ev_fork, 0));
+      } else if (is_coord_step(st) && si < first_conv) {
+        int rc = run_step(*e, st, stream);
+        if (rc) return fail(st, rc);
+        if (st.kind == StepKind::RulebookSparse) e->coord_rb[e->rulebooks[st.rulebook]->coord_out] = st.rulebook;
+        // (a submanifold table is read by the convolutions only; the others produce what later builds read)
+        if (st.kind != StepKind::RulebookSubm) SCN_HIP(hipEventRecord(e->ev_fork, stream));
       } else if (is_coord_step(st)) {
+        if (!aux_started) SCN_HIP(hipStreamWaitEvent(e->aux, e->ev_fork, 0));
+        aux_started = true;
         int rc = run_step(*e, st, e->aux);
         if (rc) return fail(st, rc);
         if (st.kind != StepKind::HashBuild) {
@@ -1693,6 +1710,8 @@ int scn_engine_forward(scn_engine* e, void* stream_) {
         }
       } else if (st.kind == StepKind::Dense && si < e->dense_maps.size() && e->dense_maps[si].p &&
                  e->dense_precleared[si] == 2) {
+        if (!aux_started) SCN_HIP(hipStreamWaitEvent(e->aux, e->ev_fork, 0));
+        aux_started = true;
         const CoordSet& cs = e->coords[e->tensors[st.t_in].coord];
         int rc = scatter_dense_build_map(cs.idx, cs.n_bound, cs.n_dev, st.dense_shape, st.has_perm ? st.perm : nullptr,
                                          e->dense_maps[si].as<int32_t>(), true, e->aux);
@@ -1700,6 +1719,7 @@ int scn_engine_forward(scn_engine* e, void* stream_) {
         e->map_built[si] = 1;
       }
     }
+    if (!aux_started) SCN_HIP(hipStreamWaitEvent(e->aux, e->ev_fork, 0));
     SCN_HIP(hipEventRecord(e->ev_join, e->aux));
     // pass 2: the feature kernels
     for (size_t si = 0; si < e->steps.size(); ++si) {
