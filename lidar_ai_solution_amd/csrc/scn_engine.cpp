@@ -1737,15 +1737,30 @@ int scn_engine_forward(scn_engine* e, void* stream_) {
         SCN_HIP(hipStreamWaitEvent(stream, e->ev_join, 0));  // row maps come after every rulebook
         waited_seq = aux_seq + 1;
       } else if (rb >= 0 && e->rb_seq[rb] > waited_seq) {
-        SCN_HIP(hipStreamWaitEvent(stream, e->rb_ready[rb], 0));
-        waited_seq = e->rb_seq[rb];
+        // A wait on the other stream costs ~2 us even when its event has long fired.  The table of a strided
+        // convolution is followed on the auxiliary stream by the submanifold table of its output
+        // coordinates, and the layers that use that one come next: one wait covers both.
+        int target = rb;
+        if (!e->rulebooks[rb]->subm)
+          for (size_t r2 = 0; r2 < e->rb_seq.size(); ++r2)
+            if (e->rb_seq[r2] == e->rb_seq[rb] + 1 && e->rulebooks[r2]->subm &&
+                e->rulebooks[r2]->coord_in == e->rulebooks[rb]->coord_out)
+              target = (int)r2;
+        if (e->rb_seq[target] == aux_seq) {
+          // the last table: what follows it on the auxiliary stream (row maps) is short; wait for all of it
+          SCN_HIP(hipStreamWaitEvent(stream, e->ev_join, 0));
+          waited_seq = aux_seq + 1;
+        } else {
+          SCN_HIP(hipStreamWaitEvent(stream, e->rb_ready[target], 0));
+          waited_seq = e->rb_seq[target];
+        }
       }
       e->dense_map_built = e->map_built[si] != 0;
       int rc = run_step(*e, st, stream);
       e->dense_map_built = false;
       if (rc) return fail(st, rc);
     }
-    SCN_HIP(hipStreamWaitEvent(stream, e->ev_join, 0));
+    if (waited_seq <= aux_seq) SCN_HIP(hipStreamWaitEvent(stream, e->ev_join, 0));
     return SCN_OK;
   }
   for (auto& st : e->steps) {
