@@ -94,8 +94,8 @@ bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* 
             }
           }
         }
-    if (!zrow.alloc(768) || hipMemset(zrow.p, 0, 512) != hipSuccess ||
-        hipMemset(zrow.as<char>() + 512, 0xFF, 256) != hipSuccess ||  // 64 words of -1 ("no neighbour")
+    if (!zrow.alloc(1536) || hipMemset(zrow.p, 0, 512) != hipSuccess ||
+        hipMemset(zrow.as<char>() + 512, 0xFF, 1024) != hipSuccess ||  // 256 words of -1 ("no neighbour")
         !wfrag32.alloc(f32.size()) || hipMemcpy(wfrag32.p, f32.data(), f32.size(), hipMemcpyHostToDevice) != hipSuccess) {
       set_error("weight upload failed");
       return false;

@@ -36,7 +36,7 @@ struct ConvArgs {
   float b_rq_s, b_rq_r;
   int relu2;
   int out_vec16;     // output rows are 16-byte aligned and a multiple of 16 bytes: 16-byte stores allowed
-  const char* zrow;  // 512 bytes of zeros (gather source of lanes without a neighbour), then 64 words of -1
+  const char* zrow;  // 512 bytes of zeros (gather source of lanes without a neighbour), then 256 words of -1
 };
 
 // Launch the kernel for these weights (one definition per element type, each in its own translation unit).

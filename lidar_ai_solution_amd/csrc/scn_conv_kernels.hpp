@@ -407,12 +407,14 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
   constexpr int NL = SLAB / 64;                  // 1 KB wave-loads per slab
   constexpr int WPT = (NL + WAVES - 1) / WAVES;  // slab loads per wave and iteration (the same for every wave:
                                                  // the waits below count loads; surplus ones go to `spare`)
-  constexpr int IDXI = G >= 2 ? G / 2 : 1;       // index loads per wave and iteration (64 entries each)
+  constexpr int IDXE = G >= 2 ? G / 2 : 1;       // index entries per wave and iteration, in units of 64
+  constexpr bool IDX4 = G >= 8;                  // 16-byte index loads (all 64 lanes busy; measured slower for G = 2, equal for 4)
+  constexpr int IDXI = IDX4 ? 1 : IDXE;          // index loads per wave and iteration
   constexpr int R = 32 * WAVES;                  // output rows per workgroup
   __shared__ v4i lds[2][SLAB];
   __shared__ v4i ring[WAVES][256];
   constexpr int DEPTH = (MT == 1 && CHUNKS <= 2) ? 2 : 4;   // index ring stages (LDS is what limits the narrow layers' occupancy)
-  __shared__ int32_t iring[DEPTH][WAVES][64 * IDXI];
+  __shared__ int32_t iring[DEPTH][WAVES][64 * IDXE];
   __shared__ v4i spare[NL % WAVES ? 64 : 1];
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -454,17 +456,27 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
                                          (lptr_t)&spare[0], 16, 0, 0);                          \
     }                                                                                           \
   }
-// neighbour rows of iteration IT -> index ring stage IT % 4: entry e = 64 q + lane is kernel offset
-// e / 32 of the iteration, tile row e % 32; slots outside the volume or beyond row n read -1
+// neighbour rows of iteration IT -> index ring stage IT % DEPTH: entry e is kernel offset e / 32 of the
+// iteration, tile row e % 32; slots outside the volume or beyond row n read -1.  Lane l of load q fetches
+// entry 64 q + l; with 8 offsets per iteration (16-byte rows) one load fetches all 256 entries instead,
+// lane l the 16 bytes of rows 4 (l % 8) .. + 3 of offset l / 8, which relies on the rulebooks' guarantee
+// that the table holds -1 for the rows between the count and the next multiple of 32.
 #define SCN_INDEX(IT)                                                                           \
   {                                                                                             \
-    _Pragma("unroll") for (int q = 0; q < IDXI; ++q) {                                          \
-      const int e_ = q * 64 + lane;                                                             \
-      const int k_ = IPO > 1 ? (IT) / IPO + e_ / 32 : (IT) * G + e_ / 32;                       \
-      const uint32_t r_ = row0 + (e_ & 31);                                                     \
-      const bool ok_ = (IT) < iters && k_ < a.kvol && r_ < n;                                   \
-      const int32_t* p_ = ok_ ? a.nbr + (size_t)k_ * a.nbr_ld + r_ : minus1 + lane;             \
-      __builtin_amdgcn_global_load_lds((gptr_t)p_, (lptr_t)&iring[(IT) & (DEPTH - 1)][wave][q * 64], 4, 0, 0); \
+    if constexpr (IDX4) {                                                                       \
+      const int k_ = (IT) * G + lane / 8;                                                       \
+      const bool ok_ = (IT) < iters && k_ < a.kvol && row0 < n;                                 \
+      const int32_t* p_ = ok_ ? a.nbr + (size_t)k_ * a.nbr_ld + row0 + 4 * (lane & 7) : minus1 + 4 * lane; \
+      __builtin_amdgcn_global_load_lds((gptr_t)p_, (lptr_t)&iring[(IT) & (DEPTH - 1)][wave][0], 16, 0, 0); \
+    } else {                                                                                    \
+      _Pragma("unroll") for (int q = 0; q < IDXI; ++q) {                                        \
+        const int e_ = q * 64 + lane;                                                           \
+        const int k_ = IPO > 1 ? (IT) / IPO + e_ / 32 : (IT) * G + e_ / 32;                     \
+        const uint32_t r_ = row0 + (e_ & 31);                                                   \
+        const bool ok_ = (IT) < iters && k_ < a.kvol && r_ < n;                                 \
+        const int32_t* p_ = ok_ ? a.nbr + (size_t)k_ * a.nbr_ld + r_ : minus1 + lane;           \
+        __builtin_amdgcn_global_load_lds((gptr_t)p_, (lptr_t)&iring[(IT) & (DEPTH - 1)][wave][q * 64], 4, 0, 0); \
+      }                                                                                         \
     }                                                                                           \
   }
 // gathers of iteration IT (neighbour rows GI[4] of this lane's slots) into the wave's stage; element
@@ -483,7 +495,7 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
 // e / SEG of the stage (e = 64 q + l), i.e. a fixed stride of 64 / SEG entries between slots.
 #define SCN_READ_INDEX(STG, GI)                                                                 \
   {                                                                                             \
-    const uint32_t base_ = iring_addr + (uint32_t)(STG) * (WAVES * 64 * IDXI * 4);              \
+    const uint32_t base_ = iring_addr + (uint32_t)(STG) * (WAVES * 64 * IDXE * 4);              \
     asm volatile("ds_read_b32 %0, %4\n\tds_read_b32 %1, %4 offset:%5\n\tds_read_b32 %2, %4 offset:%6\n\t" \
                  "ds_read_b32 %3, %4 offset:%7\n\ts_waitcnt lgkmcnt(0)"                         \
                  : "=&v"(GI[0]), "=&v"(GI[1]), "=&v"(GI[2]), "=&v"(GI[3])                       \

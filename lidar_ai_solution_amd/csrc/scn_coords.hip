@@ -330,7 +330,13 @@ __global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_
     }
     if (n_host) *n_host = n;  // pinned host word: the row count as a launch hint for the next forward
   }
-  if (o >= n) return;
+  if (o >= n) {
+    // the convolution kernels fetch table entries four rows at a time within a 32-row tile: the rows
+    // between the count and the next multiple of 32 read as "no neighbour"
+    if (o < ((n + 31u) & ~31u))
+      for (int k = 0; k < g.ks[1] * g.ks[2]; ++k) nbr[(size_t)(blockIdx.y * g.ks[1] * g.ks[2] + k) * ld + o] = -1;
+    return;
+  }
   const int k0 = blockIdx.y;
   const int4 c = out_coords[o];
   const int i0 = c.y * g.st[0] - g.pd[0] + k0 * g.dl[0];
@@ -657,9 +663,11 @@ int Rulebook::build_inverse(const Rulebook& fwd, const uint32_t* n_in_dev, hipSt
   n_bound_in = fwd.n_bound_out;
   n_bound_out = fwd.n_bound_in;
   // every offset's row of the table, up to the row bound, starts as "no neighbour"
-  if (n_bound_out)
-    hipLaunchKernelGGL(k_fill_table_rows, dim3(ceil_div(n_bound_out, 256), geom.kvol), dim3(256), 0, stream,
-                       nbr.as<int32_t>(), ld, n_bound_out, -1);
+  // (and the rows up to the next multiple of 32, which the convolution kernels may fetch)
+  const uint32_t fill_rows = std::min((n_bound_out + 31u) & ~31u, ld);
+  if (fill_rows)
+    hipLaunchKernelGGL(k_fill_table_rows, dim3(ceil_div(fill_rows, 256), geom.kvol), dim3(256), 0, stream,
+                       nbr.as<int32_t>(), ld, fill_rows, -1);
   const uint32_t blocks = n_bound_in ? ceil_div(n_bound_in, 256) : 1;  // one block even when empty: it publishes the count
   hipLaunchKernelGGL(k_invert_nbr, dim3(blocks, geom.kvol), dim3(256), 0, stream, fwd.nbr.as<int32_t>(), fwd.ld,
                      fwd.n_out_dev(), fwd.n_bound_out, nbr.as<int32_t>(), ld, n_in_dev, n_bound_out,
