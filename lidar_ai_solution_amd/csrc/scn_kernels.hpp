@@ -52,7 +52,8 @@ struct Rulebook {
   ConvGeom geom{};
   CoordTable own_in_table;    // hash of the input rows when no shared lookup is passed
   CoordLookup in_lookup;      // what the last build used to find input rows
-  DevBuf nbr;                 // int32 [kvol_cap][ld]
+  DevBuf nbr;                 // int32 [kvol_cap][ld]; every build leaves -1 in the rows from the count up to the
+                              // next multiple of 32 (the convolution kernels fetch whole 32-row tiles of entries)
   uint32_t ld = 0;
   DevBuf out_idx;             // int32 [max_out][4] (strided)
   DevBuf counters;            // uint32: [0] n_out kept, [1] n_out before truncation, [2..] scratch
