@@ -392,10 +392,18 @@ struct Mma32<1> {
 // The memory counter retires loads in order, so "at most N outstanding" names exactly which older load
 // has landed.  Issue order per iteration i: slab S(i+1), indices I(i+4), gathers G(i+1).
 // waves per SIMD the kernel is compiled for: two 8-wave workgroups per CU, or one of 10 / 12 waves
-constexpr int conv_lds_min_waves(int waves) { return waves <= 8 ? 4 : 3; }
+// (64 output channels: three 8-wave workgroups per CU, 80 registers; 181,613 rows of the benchmark frame
+// are 5,676 tiles, which two workgroups per CU (4,096 tiles) hold only in two rounds)
+// The variants that do (64- and 128-byte input rows) fit 80 registers without spilling.
+constexpr bool conv_lds_three_groups(int chunks, int mt, int waves) {
+  return mt == 2 && waves == 8 && (chunks == 4 || chunks == 8);
+}
+constexpr int conv_lds_min_waves(int chunks, int mt, int waves) {
+  return conv_lds_three_groups(chunks, mt, waves) ? 6 : waves <= 8 ? 4 : 3;
+}
 
 template <int EL, int CHUNKS, int MT, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_lds(const ConvArgs a) {
+__global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) void k_conv_lds(const ConvArgs a) {
   using Acc = typename Mma32<EL>::Acc;
   using Acc4 = typename Mma32<EL>::Acc4;
   constexpr int THREADS = 64 * WAVES;
@@ -413,7 +421,7 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
   constexpr int R = 32 * WAVES;                  // output rows per workgroup
   __shared__ v4i lds[2][SLAB];
   __shared__ v4i ring[WAVES][256];
-  constexpr int DEPTH = (MT == 1 && CHUNKS <= 2) ? 2 : 4;   // index ring stages (LDS is what limits the narrow layers' occupancy)
+  constexpr int DEPTH = ((MT == 1 && CHUNKS <= 2) || conv_lds_three_groups(CHUNKS, MT, WAVES)) ? 2 : 4;   // index ring stages (LDS is what limits the narrow layers' occupancy)
   __shared__ int32_t iring[DEPTH][WAVES][64 * IDXE];
   __shared__ v4i spare[NL % WAVES ? 64 : 1];
   const int tid = threadIdx.x;
@@ -579,7 +587,7 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(WAVES)) void k_conv_
     SCN_READ_INDEX((it + 1) & (DEPTH - 1), gi);
     SCN_GATHER(it + 1, gi);
     const uint32_t la = lds_a_addr + (uint32_t)(it & 1) * (SLAB * 16);
-    if constexpr (MT >= 4 && conv_lds_min_waves(WAVES) >= 4) {
+    if constexpr ((MT >= 4 && conv_lds_min_waves(CHUNKS, MT, WAVES) >= 4) || conv_lds_three_groups(CHUNKS, MT, WAVES)) {
       // 64 accumulator registers leave room for one set of fragments under the 128-register budget of
       // four waves per SIMD (a spill would also put scratch loads into the memory counter and break the
       // counts above); the other three waves of the SIMD cover the LDS latency instead
