@@ -303,14 +303,17 @@ def test_fp16_conv_within_tolerance(cin, cout, centerpoint_input):
     assert np.allclose(out.cpu().numpy().astype(np.float32), ref, rtol=2e-3, atol=1e-3)
 
 
-def test_fused_residual_epilogue_matches_unfused_oracle(centerpoint_input):
-    """conv2 -> Add(identity) -> ReLU fused into one kernel equals the node-by-node oracle."""
+@pytest.mark.parametrize("channels,n_rows", [(32, 20000), (64, 9991), (128, 5003), (16, 4097)])
+def test_fused_residual_epilogue_matches_unfused_oracle(channels, n_rows, centerpoint_input):
+    """conv2 -> Add(identity) -> ReLU fused into one kernel equals the node-by-node oracle, for every tile
+    width of the kernel (the residual is staged per tile from 64 channels up) and row counts that end inside a tile."""
     _, idx_all = centerpoint_input
     rng = np.random.default_rng(21)
-    idx = idx_all[:20000]
+    idx = idx_all[:n_rows]
     n = idx.shape[0]
     grid = (41, 1440, 1440)
-    cin = cout = 32
+    cin = cout = channels
+    note(f"fused residual epilogue, {channels} channels, {n} rows")
     x = rng.integers(-127, 128, (n, cin)).astype(np.int8)
     ident = rng.integers(0, 128, (n, cout)).astype(np.int8)
     w, b, ranges = _weights(rng, cout, (3, 3, 3), cin)
@@ -328,6 +331,12 @@ def test_fused_residual_epilogue_matches_unfused_oracle(centerpoint_input):
     out, _ = conv.forward(rb, to_dev(x), n, x_range=x_range, relu=False, out_int8=True, out_range=out_range,
                           res=to_dev(ident), res_range=res_range, mid_int8=True, mid_range=mid_range, relu2=True)
     assert np.array_equal(out.cpu().numpy(), want)
+    note("the same with the convolution's own ReLU in front of the intermediate quantiser, no ReLU after the add")
+    mid_r = O.epilogue(acc_ref, scale, b.astype(np.float32), True, True, mid_range)
+    want_r = O.add(mid_r, mid_range, ident, res_range, False, True, out_range)
+    out_r, _ = conv.forward(rb, to_dev(x), n, x_range=x_range, relu=True, out_int8=True, out_range=out_range,
+                            res=to_dev(ident), res_range=res_range, mid_int8=True, mid_range=mid_range, relu2=False)
+    assert np.array_equal(out_r.cpu().numpy(), want_r)
     note("fp16-stored conv output and fp16 identity, int8 add re-quantising both, int8 out")
     ident16 = (rng.standard_normal((n, cout)) * 2).astype(np.float16)
     mid16 = O.epilogue(acc_ref, scale, b.astype(np.float32), False, False)
