@@ -386,15 +386,15 @@ struct Mma32<1> {
 //   iteration     = 4 K-steps = 4 KB of gathered rows per wave (32 rows x 8 chunks, or G = 8 / SEG
 //                   kernel offsets of SEG-chunk rows) and a weight slab of 4 * MT fragments
 //   LDS           = 2 weight slabs (iteration i, i+1), one 4 KB stage of gathered rows per wave, and a
-//                   4-deep ring of neighbour indices per wave (they always miss the caches)
+//                   ring of neighbour indices per wave, DEPTH = 4 or 2 iterations deep (they always miss the caches)
 //   per iteration = one barrier for the slab; a wave consumes only rows and indices it fetched itself,
 //                   so those need a wait on the wave's own memory counter only
 // The memory counter retires loads in order, so "at most N outstanding" names exactly which older load
-// has landed.  Issue order per iteration i: slab S(i+1), indices I(i+4), gathers G(i+1).
-// waves per SIMD the kernel is compiled for: two 8-wave workgroups per CU, or one of 10 / 12 waves
-// (64 output channels: three 8-wave workgroups per CU, 80 registers; 181,613 rows of the benchmark frame
-// are 5,676 tiles, which two workgroups per CU (4,096 tiles) hold only in two rounds)
-// The variants that do (64- and 128-byte input rows) fit 80 registers without spilling.
+// has landed.  Issue order per iteration i: slab S(i+1), indices I(i+DEPTH), gathers G(i+1).
+// Waves per SIMD the kernel is compiled for: two 8-wave workgroups per CU (128 registers), or one of
+// 9 .. 12 waves.  The 64-channel kernels with 64- and 128-byte input rows take three 8-wave workgroups per
+// CU instead (80 registers without spilling, with a two-stage index ring and one set of A fragments): a
+// lidar frame's 64-channel stage is more tiles than two workgroups per CU hold in one round.
 constexpr bool conv_lds_three_groups(int chunks, int mt, int waves) {
   return mt == 2 && waves == 8 && (chunks == 4 || chunks == 8);
 }
@@ -551,7 +551,7 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
                                 ((2 * ((SS) % (SEG / 2 > 0 ? SEG / 2 : 1))) ^ (SW))) * 16       \
             : (BB) + (uint32_t)(2 * (SS) * 32) * 16)
 
-  // prologue: indices of iterations 0..3, slab 0, then the gathers of iteration 0
+  // prologue: indices of iterations 0 .. DEPTH-1, slab 0, then the gathers of iteration 0
   SCN_INDEX(0);
   SCN_INDEX(1);
   if constexpr (DEPTH == 4) {
