@@ -560,12 +560,22 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
   }
   SCN_SLAB(0);
   SCN_WAIT_VM((DEPTH - 1) * IDXI + WPT);  // I(0), the oldest, has landed
+  // A wave whose 32 rows have no neighbour at any kernel offset of an iteration (rows of one z slice and
+  // the offsets that leave it, tiles next to empty space: a third to a half of all (tile, offset)
+  // combinations of a lidar frame) skips that iteration's gathers, operand reads and MFMAs -- they would
+  // add zeros -- and only takes its part in the slab loads and the barrier.
+  bool work;  // wave-uniform: the current iteration has at least one neighbour row
   {
     int32_t gi[4];
     SCN_READ_INDEX(0, gi);
-    SCN_GATHER(0, gi);
+    work = __builtin_amdgcn_ballot_w64((gi[0] & gi[1] & gi[2] & gi[3]) >= 0) != 0;
+    if (work) {
+      SCN_GATHER(0, gi);
+      SCN_WAIT_VM(4);  // ... and this wave's part of S(0) (younger: G(0))
+    } else {
+      SCN_WAIT_VM(0);
+    }
   }
-  SCN_WAIT_VM(4);  // ... and this wave's part of S(0) (younger: G(0))
   asm volatile("s_barrier" ::: "memory");
 
   for (int it = 0; it < iters; ++it) {
@@ -574,7 +584,7 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
     SCN_WAIT_VM(WPT + IDXI);  // G(it), I(it+1) and everything older have landed
     v4i bf[4];
     int32_t gi[4];
-    {
+    if (work) {
       uint32_t bb = b_base, sw = b_swz;
       asm volatile("" : "+v"(bb), "+v"(sw));  // keeps the four addresses out of loop-carried registers
       asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\tds_read_b128 %3, %7"
@@ -585,8 +595,11 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
     }
     // waits for the index reads and, LDS returning in order, for bf[]: the stage may be overwritten
     SCN_READ_INDEX((it + 1) & (DEPTH - 1), gi);
-    SCN_GATHER(it + 1, gi);
+    // (iterations past the end read -1 everywhere)
+    const bool work_next = __builtin_amdgcn_ballot_w64((gi[0] & gi[1] & gi[2] & gi[3]) >= 0) != 0;
+    if (work_next) SCN_GATHER(it + 1, gi);
     const uint32_t la = lds_a_addr + (uint32_t)(it & 1) * (SLAB * 16);
+    if (work) {
     if constexpr ((MT >= 4 && conv_lds_min_waves(CHUNKS, MT, WAVES) >= 4) || conv_lds_three_groups(CHUNKS, MT, WAVES)) {
       // 64 accumulator registers leave room for one set of fragments under the 128-register budget of
       // four waves per SIMD (a spill would also put scratch loads into the memory counter and break the
@@ -618,7 +631,14 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
 #pragma unroll
       for (int t = 0; t < MT; ++t) acc[t] = Mma32<EL>::run(afB[t], bf[3], acc[t]);
     }
-    SCN_WAIT_VM(4);  // this wave's part of S(it+1) has landed (younger: G(it+1))
+    }
+    // this wave's part of S(it+1) has landed (younger: G(it+1), when it was issued)
+    if (work_next) {
+      SCN_WAIT_VM(4);
+    } else {
+      SCN_WAIT_VM(0);
+    }
+    work = work_next;
     // every wave has read slab it (its fragments are in registers) and written its part of slab it+1
     asm volatile("s_barrier" ::: "memory");
   }
