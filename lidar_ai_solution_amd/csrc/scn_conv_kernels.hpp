@@ -402,8 +402,14 @@ constexpr int conv_lds_min_waves(int chunks, int mt, int waves) {
   return conv_lds_three_groups(chunks, mt, waves) ? 6 : waves <= 8 ? 4 : 3;
 }
 
-template <int EL, int CHUNKS, int MT, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) void k_conv_lds(const ConvArgs a) {
+// AHEAD = iterations between the issue of an iteration's gathers / weight slab and their use.  1: one stage per
+// wave and two slab buffers, which is what fits the LDS of full CUs, and the only value the dispatch below
+// instantiates.  2: three of each, meant for launches of few rows (at most four 32-row tiles per CU), where
+// nothing competes for the CU and an iteration lasts as long as the round trip of its gathers (about 1 us
+// whatever the layer's width).  NOT DISPATCHED: its first run on the GPU ended in a memory fault whose cause
+// has not been found by reading the code and its assembly; it must not be instantiated before it is.
+template <int EL, int CHUNKS, int MT, int WAVES, int AHEAD = 1>
+__global__ __launch_bounds__(64 * WAVES, AHEAD > 1 ? 2 : conv_lds_min_waves(CHUNKS, MT, WAVES)) void k_conv_lds(const ConvArgs a) {
   using Acc = typename Mma32<EL>::Acc;
   using Acc4 = typename Mma32<EL>::Acc4;
   constexpr int THREADS = 64 * WAVES;
@@ -419,9 +425,12 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
   constexpr bool IDX4 = G >= 8;                  // 16-byte index loads (all 64 lanes busy; measured slower for G = 2, equal for 4)
   constexpr int IDXI = IDX4 ? 1 : IDXE;          // index loads per wave and iteration
   constexpr int R = 32 * WAVES;                  // output rows per workgroup
-  __shared__ v4i lds[2][SLAB];
-  __shared__ v4i ring[WAVES][256];
-  constexpr int DEPTH = ((MT == 1 && CHUNKS <= 2) || conv_lds_three_groups(CHUNKS, MT, WAVES)) ? 2 : 4;   // index ring stages (LDS is what limits the narrow layers' occupancy)
+  constexpr int NBUF = AHEAD + 1;                // slab buffers, and stages of gathered rows per wave
+  constexpr int NST = AHEAD > 1 ? NBUF : 1;
+  __shared__ v4i lds[NBUF][SLAB];
+  __shared__ v4i ring[WAVES][NST][256];
+  constexpr int DEPTH = AHEAD > 1 ? 4 : ((MT == 1 && CHUNKS <= 2) || conv_lds_three_groups(CHUNKS, MT, WAVES)) ? 2 : 4;   // index ring stages (LDS is what limits the narrow layers' occupancy)
+  static_assert(AHEAD >= 1 && AHEAD < DEPTH, "the index ring must reach past the gathers in flight");
   __shared__ int32_t iring[DEPTH][WAVES][64 * IDXE];
   __shared__ v4i spare[NL % WAVES ? 64 : 1];
   const int tid = threadIdx.x;
@@ -451,14 +460,14 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
 // after EVERY outstanding global_load_lds (vmcnt(0)), which would drain the loads issued for the next
 // iterations.  The waits that are really needed are the explicit ones below.
 // weight slab of iteration IT -> LDS buffer IT % 2 (iterations past the end re-load the last slab)
-#define SCN_SLAB(IT)                                                                            \
+#define SCN_SLAB(IT, BUF)                                                                       \
   {                                                                                             \
     const int it_ = (IT) < iters ? (IT) : iters - 1;                                            \
     _Pragma("unroll") for (int j = 0; j < WPT; ++j) {                                           \
       const int f_ = j * WAVES + wave; /* wave-uniform */                                       \
       if (NL % WAVES == 0 || f_ < NL)                                                           \
         __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + (size_t)it_ * SLAB + f_ * 64 + lane),  \
-                                         (lptr_t)&lds[(IT) & 1][f_ * 64], 16, 0, 0);            \
+                                         (lptr_t)&lds[BUF][f_ * 64], 16, 0, 0);                 \
       else                                                                                      \
         __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + (size_t)it_ * SLAB + lane),            \
                                          (lptr_t)&spare[0], 16, 0, 0);                          \
@@ -489,14 +498,14 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
   }
 // gathers of iteration IT (neighbour rows GI[4] of this lane's slots) into the wave's stage; element
 // e = 64 q + lane of its [G][32 rows][SEG] array
-#define SCN_GATHER(IT, GI)                                                                      \
+#define SCN_GATHER(IT, GI, STG)                                                                 \
   {                                                                                             \
     _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                             \
       const int e_ = q * 64 + lane;                                                             \
       const int row_ = (e_ / SEG) % 32;                                                         \
       const int cg_ = (IPO > 1 ? ((IT) % IPO) * 8 : 0) + ((e_ % SEG) ^ ((row_ / RP) % SEG));    \
       const char* p_ = GI[q] >= 0 ? xb + (size_t)(uint32_t)GI[q] * ldb + cg_ * 16 : zrow + cg_ * 16; \
-      __builtin_amdgcn_global_load_lds((gptr_t)p_, (lptr_t)&ring[wave][q * 64], 16, 0, 0);      \
+      __builtin_amdgcn_global_load_lds((gptr_t)p_, (lptr_t)&ring[wave][STG][q * 64], 16, 0, 0); \
     }                                                                                           \
   }
 // this lane's four index slots of ring stage STG -> GI[4], waited for.  Slot q of lane l is entry
@@ -539,7 +548,7 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
       asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(AF[0]) : "n"(KEEP) : "memory");               \
   }
 
-  const uint32_t ring_addr = (uint32_t)(uintptr_t)(lptr_t)&ring[wave][0];
+  const uint32_t ring_addr = (uint32_t)(uintptr_t)(lptr_t)&ring[wave][0][0];
   const uint32_t iring_addr = (uint32_t)(uintptr_t)(lptr_t)&iring[0][wave][0] + (uint32_t)(lane / SEG) * 4;
   const uint32_t lds_a_addr = (uint32_t)(uintptr_t)(lptr_t)&lds[0][lane];
   // B-operand read address of K-step ss inside the wave's stage: row ln, chunk 2 ss' + lh at its swizzled
@@ -551,59 +560,23 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
                                 ((2 * ((SS) % (SEG / 2 > 0 ? SEG / 2 : 1))) ^ (SW))) * 16       \
             : (BB) + (uint32_t)(2 * (SS) * 32) * 16)
 
-  // prologue: indices of iterations 0 .. DEPTH-1, slab 0, then the gathers of iteration 0
-  SCN_INDEX(0);
-  SCN_INDEX(1);
-  if constexpr (DEPTH == 4) {
-    SCN_INDEX(2);
-    SCN_INDEX(3);
+  // B fragments of the wave's stage STG (the four K-steps of an iteration)
+#define SCN_READ_B(STG, BF)                                                                     \
+  {                                                                                             \
+    uint32_t bb = b_base + (uint32_t)(STG) * 4096u, sw = b_swz;                                 \
+    asm volatile("" : "+v"(bb), "+v"(sw)); /* keeps the four addresses out of loop-carried registers */ \
+    asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\tds_read_b128 %3, %7" \
+                 : "=&v"(BF[0]), "=&v"(BF[1]), "=&v"(BF[2]), "=&v"(BF[3])                       \
+                 : "v"(SCN_B_ADDR(0, bb, sw)), "v"(SCN_B_ADDR(1, bb, sw)), "v"(SCN_B_ADDR(2, bb, sw)), \
+                   "v"(SCN_B_ADDR(3, bb, sw))                                                   \
+                 : "memory");                                                                   \
   }
-  SCN_SLAB(0);
-  SCN_WAIT_VM((DEPTH - 1) * IDXI + WPT);  // I(0), the oldest, has landed
-  // A wave whose 32 rows have no neighbour at any kernel offset of an iteration (rows of one z slice and
-  // the offsets that leave it, tiles next to empty space: a third to a half of all (tile, offset)
-  // combinations of a lidar frame) skips that iteration's gathers, operand reads and MFMAs -- they would
-  // add zeros -- and only takes its part in the slab loads and the barrier.
-  bool work;  // wave-uniform: the current iteration has at least one neighbour row
-  {
-    int32_t gi[4];
-    SCN_READ_INDEX(0, gi);
-    work = __builtin_amdgcn_ballot_w64((gi[0] & gi[1] & gi[2] & gi[3]) >= 0) != 0;
-    if (work) {
-      SCN_GATHER(0, gi);
-      SCN_WAIT_VM(4);  // ... and this wave's part of S(0) (younger: G(0))
-    } else {
-      SCN_WAIT_VM(0);
-    }
-  }
-  asm volatile("s_barrier" ::: "memory");
-
-  for (int it = 0; it < iters; ++it) {
-    SCN_SLAB(it + 1);
-    SCN_INDEX(it + DEPTH);
-    SCN_WAIT_VM(WPT + IDXI);  // G(it), I(it+1) and everything older have landed
-    v4i bf[4];
-    int32_t gi[4];
-    if (work) {
-      uint32_t bb = b_base, sw = b_swz;
-      asm volatile("" : "+v"(bb), "+v"(sw));  // keeps the four addresses out of loop-carried registers
-      asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\tds_read_b128 %3, %7"
-                   : "=&v"(bf[0]), "=&v"(bf[1]), "=&v"(bf[2]), "=&v"(bf[3])
-                   : "v"(SCN_B_ADDR(0, bb, sw)), "v"(SCN_B_ADDR(1, bb, sw)), "v"(SCN_B_ADDR(2, bb, sw)),
-                     "v"(SCN_B_ADDR(3, bb, sw))
-                   : "memory");
-    }
-    // waits for the index reads and, LDS returning in order, for bf[]: the stage may be overwritten
-    SCN_READ_INDEX((it + 1) & (DEPTH - 1), gi);
-    // (iterations past the end read -1 everywhere)
-    const bool work_next = __builtin_amdgcn_ballot_w64((gi[0] & gi[1] & gi[2] & gi[3]) >= 0) != 0;
-    if (work_next) SCN_GATHER(it + 1, gi);
-    const uint32_t la = lds_a_addr + (uint32_t)(it & 1) * (SLAB * 16);
-    if (work) {
-    if constexpr ((MT >= 4 && conv_lds_min_waves(CHUNKS, MT, WAVES) >= 4) || conv_lds_three_groups(CHUNKS, MT, WAVES)) {
+  // the 4 * MT MFMAs of an iteration: A fragments from the slab at LDS address la, B fragments bf[]
+  auto multiply = [&](const uint32_t la, const v4i (&bf)[4]) {
+    if constexpr (AHEAD == 1 && ((MT >= 4 && conv_lds_min_waves(CHUNKS, MT, WAVES) >= 4) || conv_lds_three_groups(CHUNKS, MT, WAVES))) {
       // 64 accumulator registers leave room for one set of fragments under the 128-register budget of
       // four waves per SIMD (a spill would also put scratch loads into the memory counter and break the
-      // counts above); the other three waves of the SIMD cover the LDS latency instead
+      // counts below); the other three waves of the SIMD cover the LDS latency instead
       v4i af[MT];
 #pragma unroll
       for (int ss = 0; ss < 4; ++ss) {
@@ -631,17 +604,107 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
 #pragma unroll
       for (int t = 0; t < MT; ++t) acc[t] = Mma32<EL>::run(afB[t], bf[3], acc[t]);
     }
+  };
+
+  // A wave whose 32 rows have no neighbour at any kernel offset of an iteration (rows of one z slice and
+  // the offsets that leave it, tiles next to empty space: a third to a half of all (tile, offset)
+  // combinations of a synthetic frame, a tenth of a real one's) skips that iteration's operand reads and
+  // MFMAs -- they would add zeros -- and, where the waits below can follow it, its gathers.
+  if constexpr (AHEAD == 1) {
+    // prologue: indices of iterations 0 .. DEPTH-1, slab 0, then the gathers of iteration 0
+    SCN_INDEX(0);
+    SCN_INDEX(1);
+    if constexpr (DEPTH == 4) {
+      SCN_INDEX(2);
+      SCN_INDEX(3);
     }
-    // this wave's part of S(it+1) has landed (younger: G(it+1), when it was issued)
-    if (work_next) {
-      SCN_WAIT_VM(4);
-    } else {
-      SCN_WAIT_VM(0);
+    SCN_SLAB(0, 0);
+    SCN_WAIT_VM((DEPTH - 1) * IDXI + WPT);  // I(0), the oldest, has landed
+    bool work;  // wave-uniform: the current iteration has at least one neighbour row
+    {
+      int32_t gi[4];
+      SCN_READ_INDEX(0, gi);
+      work = __builtin_amdgcn_ballot_w64((gi[0] & gi[1] & gi[2] & gi[3]) >= 0) != 0;
+      if (work) {
+        SCN_GATHER(0, gi, 0);
+        SCN_WAIT_VM(4);  // ... and this wave's part of S(0) (younger: G(0))
+      } else {
+        SCN_WAIT_VM(0);
+      }
     }
-    work = work_next;
-    // every wave has read slab it (its fragments are in registers) and written its part of slab it+1
     asm volatile("s_barrier" ::: "memory");
+
+    for (int it = 0; it < iters; ++it) {
+      SCN_SLAB(it + 1, (it + 1) & 1);
+      SCN_INDEX(it + DEPTH);
+      SCN_WAIT_VM(WPT + IDXI);  // G(it), I(it+1) and everything older have landed
+      v4i bf[4];
+      int32_t gi[4];
+      if (work) SCN_READ_B(0, bf);
+      // waits for the index reads and, LDS returning in order, for bf[]: the stage may be overwritten
+      SCN_READ_INDEX((it + 1) & (DEPTH - 1), gi);
+      // (iterations past the end read -1 everywhere)
+      const bool work_next = __builtin_amdgcn_ballot_w64((gi[0] & gi[1] & gi[2] & gi[3]) >= 0) != 0;
+      if (work_next) SCN_GATHER(it + 1, gi, 0);
+      if (work) multiply(lds_a_addr + (uint32_t)(it & 1) * (SLAB * 16), bf);
+      // this wave's part of S(it+1) has landed (younger: G(it+1), when it was issued)
+      if (work_next) {
+        SCN_WAIT_VM(4);
+      } else {
+        SCN_WAIT_VM(0);
+      }
+      work = work_next;
+      // every wave has read slab it (its fragments are in registers) and written its part of slab it+1
+      asm volatile("s_barrier" ::: "memory");
+    }
+  } else {
+    // Loads of one iteration, in issue order: S (WPT), I (IDXI) at its top, G (4) in its middle; the gathers
+    // are issued for every iteration here (empty ones fetch the row of zeros) so that the counts hold.
+    constexpr int PER_IT = WPT + IDXI + 4;
+    // prologue: indices 0 .. DEPTH-1, slabs and gathers 0 .. AHEAD-1, everything landed
+    SCN_INDEX(0);
+    SCN_INDEX(1);
+    SCN_INDEX(2);
+    SCN_INDEX(3);
+#pragma unroll
+    for (int j = 0; j < AHEAD; ++j) SCN_SLAB(j, j);
+    SCN_WAIT_VM((DEPTH - AHEAD) * IDXI + AHEAD * WPT);  // I(0) .. I(AHEAD-1) have landed
+    uint32_t workbits = 0;  // wave-uniform; bit j: iteration it + j has at least one neighbour row
+#pragma unroll
+    for (int j = 0; j < AHEAD; ++j) {
+      int32_t gi[4];
+      SCN_READ_INDEX(j, gi);
+      if (__builtin_amdgcn_ballot_w64((gi[0] & gi[1] & gi[2] & gi[3]) >= 0) != 0) workbits |= 1u << j;
+      SCN_GATHER(j, gi, j);
+    }
+    SCN_WAIT_VM(0);
+    asm volatile("s_barrier" ::: "memory");
+
+    uint32_t rbuf = 0;  // it % NBUF: slab buffer and stage of the current iteration
+    for (int it = 0; it < iters; ++it) {
+      const uint32_t wbuf = rbuf == 0 ? (uint32_t)AHEAD : rbuf - 1;  // (it + AHEAD) % NBUF: read last in iteration it-1
+      SCN_SLAB(it + AHEAD, wbuf);
+      SCN_INDEX(it + DEPTH);
+      // G(it) has landed: younger are S and I of this iteration and everything of iterations it-AHEAD+1 .. it-1
+      SCN_WAIT_VM((AHEAD - 1) * PER_IT + WPT + IDXI);
+      const bool work = workbits & 1u;
+      v4i bf[4];
+      int32_t gi[4];
+      if (work) SCN_READ_B(rbuf, bf);
+      // waits for the index reads and, LDS returning in order, for the B reads of this and earlier iterations
+      SCN_READ_INDEX((it + AHEAD) & (DEPTH - 1), gi);
+      workbits >>= 1;
+      if (__builtin_amdgcn_ballot_w64((gi[0] & gi[1] & gi[2] & gi[3]) >= 0) != 0) workbits |= 1u << (AHEAD - 1);
+      SCN_GATHER(it + AHEAD, gi, wbuf);
+      if (work) multiply(lds_a_addr + rbuf * (uint32_t)(SLAB * 16), bf);
+      // this wave's part of S(it+1) has landed: younger are I and G of the iteration that issued it and
+      // everything of the AHEAD-1 iterations since
+      SCN_WAIT_VM(IDXI + 4 + (AHEAD - 1) * PER_IT);
+      asm volatile("s_barrier" ::: "memory");
+      rbuf = rbuf == (uint32_t)AHEAD ? 0u : rbuf + 1;
+    }
   }
+#undef SCN_READ_B
 #undef SCN_READ_INDEX
 #undef SCN_B_ADDR
 #undef SCN_READ_A
@@ -710,7 +773,7 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
   // of the tile 16 times.  The pieces go through the wave's LDS stage instead (same XOR placement as the
   // gathers) and leave as 16 bytes per lane, 8 lanes per row.  A residual of the output's element size
   // comes in the same way first: each piece finds its 4 residual values in the slot it then overwrites.
-  char* stage = reinterpret_cast<char*>(&ring[wave][0]);
+  char* stage = reinterpret_cast<char*>(&ring[wave][0][0]);
   const bool out8 = a.out_dtype == SCN_DTYPE_INT8;
   // (16-channel rows are one 16-byte chunk: staging them costs more than the two 4-byte reads it replaces)
   const bool res_staged = a.res && a.res_vec16 && a.res_dtype == a.out_dtype && cout_pad >= 32;
@@ -820,11 +883,12 @@ static void launch_conv_rows(const ConvArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL((k_conv_rows<EL, CHUNKS, MT, NT>), dim3(blocks), dim3(256), 0, stream, a);
 }
 
-template <int EL, int CHUNKS, int MT, int WAVES>
+template <int EL, int CHUNKS, int MT, int WAVES, int AHEAD = 1>
 static void launch_conv_lds(const ConvArgs& a, hipStream_t stream) {
+  static_assert(AHEAD == 1, "the deeper load pipeline faulted on the GPU and is switched off");
   constexpr uint32_t R = 32 * WAVES;
   const uint32_t blocks = 8 * ceil_div(ceil_div(a.n_bound, R), 8);  // see xcd_tile()
-  hipLaunchKernelGGL((k_conv_lds<EL, CHUNKS, MT, WAVES>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
+  hipLaunchKernelGGL((k_conv_lds<EL, CHUNKS, MT, WAVES, AHEAD>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
 }
 
 // Workgroup size of the 128-channel kernel.  A layer of a lidar backbone's deep stages is about one
@@ -837,9 +901,14 @@ static int conv_lds_waves(uint32_t n_hint) {
     const char* e = getenv("SCN_CONV_WAVES");
     return e ? atoi(e) : 0;
   }();
-  if (forced >= 8 && forced <= 12) return forced;
+  if (forced == 2 || forced == 4 || (forced >= 8 && forced <= 12)) return forced;
   constexpr uint32_t kCus = 256;
   const uint32_t waves = ceil_div(n_hint, kCus * 32u);  // 32-row tiles per CU
+  // Few rows (a real frame's deep stages are 10,000 .. 30,000 rows): a workgroup's kernel offsets are a
+  // dependent chain whose step grows with the loads its waves issue together, and 8-wave workgroups
+  // would leave most CUs idle, so the tiles are spread over more, smaller workgroups.
+  if (waves <= 2) return 2;
+  if (waves <= 4) return 4;
   if (waves <= 8) return 8;
   if (waves <= 12) return (int)waves;
   return 8;
@@ -849,9 +918,16 @@ template <int EL, int CHUNKS>
 static bool dispatch_mt32(int mt, uint32_t n_hint, const ConvArgs& a, hipStream_t stream) {
   switch (mt) {
     case 1: launch_conv_lds<EL, CHUNKS, 1, 4>(a, stream); return true;
-    case 2: launch_conv_lds<EL, CHUNKS, 2, 8>(a, stream); return true;
+    case 2:
+      if (conv_lds_waves(n_hint) <= 4)
+        launch_conv_lds<EL, CHUNKS, 2, 4>(a, stream);
+      else
+        launch_conv_lds<EL, CHUNKS, 2, 8>(a, stream);
+      return true;
     case 4:
       switch (conv_lds_waves(n_hint)) {
+        case 2: launch_conv_lds<EL, CHUNKS, 4, 2>(a, stream); return true;
+        case 4: launch_conv_lds<EL, CHUNKS, 4, 4>(a, stream); return true;
         case 9: launch_conv_lds<EL, CHUNKS, 4, 9>(a, stream); return true;
         case 10: launch_conv_lds<EL, CHUNKS, 4, 10>(a, stream); return true;
         case 11: launch_conv_lds<EL, CHUNKS, 4, 11>(a, stream); return true;
