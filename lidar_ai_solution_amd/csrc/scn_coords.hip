@@ -313,8 +313,9 @@ __device__ __forceinline__ int32_t coord_row(const CoordLookup& lk, uint32_t key
   return table_lookup(lk.slots, lk.mask, key);
 }
 
-// nbr[k][o] = row of the input at  o*stride - pad + k*dilation  (or -1).  grid.y = k0; a thread
-// walks the K1*K2 offsets of its k0 plane (independent lookups, coalesced stores per offset).
+// nbr[k][o] = row of the input at  o*stride - pad + k*dilation  (or -1).  grid.y = (k0, k1); a thread
+// walks the K2 offsets of its line (independent lookups, coalesced stores per offset): short chains and
+// K0*K1 times the rows in threads, because the first table of a frame is on the critical path.
 // Used for both kinds: submanifold passes stride 1 and pad = floor(K/2)*dilation.
 // Thread (0,0) also publishes the row count for the kernels that follow (n_publish, nullable).
 __global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_coords, const uint32_t* n_out_dev,
@@ -330,33 +331,31 @@ __global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_
     }
     if (n_host) *n_host = n;  // pinned host word: the row count as a launch hint for the next forward
   }
+  const int k01 = blockIdx.y;  // k0 * K1 + k1
   if (o >= n) {
     // the convolution kernels fetch table entries four rows at a time within a 32-row tile: the rows
     // between the count and the next multiple of 32 read as "no neighbour"
     if (o < ((n + 31u) & ~31u))
-      for (int k = 0; k < g.ks[1] * g.ks[2]; ++k) nbr[(size_t)(blockIdx.y * g.ks[1] * g.ks[2] + k) * ld + o] = -1;
+      for (int k = 0; k < g.ks[2]; ++k) nbr[(size_t)(k01 * g.ks[2] + k) * ld + o] = -1;
     return;
   }
-  const int k0 = blockIdx.y;
+  const int k0 = k01 / g.ks[1], k1 = k01 - k0 * g.ks[1];
   const int4 c = out_coords[o];
   const int i0 = c.y * g.st[0] - g.pd[0] + k0 * g.dl[0];
-  const bool ok0 = c.x == 0 && i0 >= 0 && i0 < g.gi[0];
-  const bool centre0 = identity_center && k0 == g.ks[0] / 2;
-  for (int k1 = 0; k1 < g.ks[1]; ++k1) {
-    const int i1 = c.z * g.st[1] - g.pd[1] + k1 * g.dl[1];
-    const bool ok1 = ok0 && i1 >= 0 && i1 < g.gi[1];
-    const uint32_t line = ((uint32_t)i0 * (uint32_t)g.gi[1] + (uint32_t)i1) * (uint32_t)g.gi[2];
+  const int i1 = c.z * g.st[1] - g.pd[1] + k1 * g.dl[1];
+  const bool ok1 = c.x == 0 && i0 >= 0 && i0 < g.gi[0] && i1 >= 0 && i1 < g.gi[1];
+  const bool centre01 = identity_center && k0 == g.ks[0] / 2 && k1 == g.ks[1] / 2;
+  const uint32_t line = ((uint32_t)i0 * (uint32_t)g.gi[1] + (uint32_t)i1) * (uint32_t)g.gi[2];
 #pragma unroll 3
-    for (int k2 = 0; k2 < g.ks[2]; ++k2) {
-      const int i2 = c.w * g.st[2] - g.pd[2] + k2 * g.dl[2];
-      int32_t res = -1;
-      if (centre0 && k1 == g.ks[1] / 2 && k2 == g.ks[2] / 2) {
-        res = (int32_t)o;
-      } else if (ok1 && i2 >= 0 && i2 < g.gi[2]) {
-        res = coord_row(lk, line + (uint32_t)i2);
-      }
-      nbr[(size_t)((k0 * g.ks[1] + k1) * g.ks[2] + k2) * ld + o] = res;
+  for (int k2 = 0; k2 < g.ks[2]; ++k2) {
+    const int i2 = c.w * g.st[2] - g.pd[2] + k2 * g.dl[2];
+    int32_t res = -1;
+    if (centre01 && k2 == g.ks[2] / 2) {
+      res = (int32_t)o;
+    } else if (ok1 && i2 >= 0 && i2 < g.gi[2]) {
+      res = coord_row(lk, line + (uint32_t)i2);
     }
+    nbr[(size_t)(k01 * g.ks[2] + k2) * ld + o] = res;
   }
 }
 
@@ -455,7 +454,7 @@ int set_count(uint32_t* dst, const uint32_t* n_dev, uint32_t n_bound, hipStream_
 static int launch_build_nbr(const Rulebook& rb, const int32_t* out_coords, const uint32_t* n_dev, uint32_t n_bound,
                             bool identity_center, uint32_t* n_publish, hipStream_t stream) {
   const uint32_t blocks = n_bound ? ceil_div(n_bound, 256) : 1;  // one block even when empty: it publishes the count
-  hipLaunchKernelGGL(k_build_nbr, dim3(blocks, rb.geom.ks[0]), dim3(256), 0, stream, (const int4*)out_coords, n_dev,
+  hipLaunchKernelGGL(k_build_nbr, dim3(blocks, rb.geom.ks[0] * rb.geom.ks[1]), dim3(256), 0, stream, (const int4*)out_coords, n_dev,
                      n_bound, to_dev(rb.geom), rb.in_lookup, rb.nbr.as<int32_t>(), rb.ld, identity_center ? 1 : 0,
                      n_publish, rb.host_count.as<uint32_t>());
   SCN_HIP(hipGetLastError());
