@@ -399,7 +399,7 @@ constexpr bool conv_lds_three_groups(int chunks, int mt, int waves) {
   return mt == 2 && waves == 8 && (chunks == 4 || chunks == 8);
 }
 constexpr int conv_lds_min_waves(int chunks, int mt, int waves) {
-  return conv_lds_three_groups(chunks, mt, waves) ? 6 : waves <= 8 ? 4 : 3;
+  return conv_lds_three_groups(chunks, mt, waves) ? 6 : (mt >= 2 && waves <= 4) ? 2 : waves <= 8 ? 4 : 3;
 }
 
 // AHEAD = iterations between the issue of an iteration's gathers / weight slab and their use.  1: one stage per
@@ -573,10 +573,11 @@ __global__ __launch_bounds__(64 * WAVES, AHEAD > 1 ? 2 : conv_lds_min_waves(CHUN
   }
   // the 4 * MT MFMAs of an iteration: A fragments from the slab at LDS address la, B fragments bf[]
   auto multiply = [&](const uint32_t la, const v4i (&bf)[4]) {
-    if constexpr (AHEAD == 1 && ((MT >= 4 && conv_lds_min_waves(CHUNKS, MT, WAVES) >= 4) || conv_lds_three_groups(CHUNKS, MT, WAVES))) {
+    if constexpr (AHEAD == 1 && WAVES >= 8 && ((MT >= 4 && conv_lds_min_waves(CHUNKS, MT, WAVES) >= 4) || conv_lds_three_groups(CHUNKS, MT, WAVES))) {
       // 64 accumulator registers leave room for one set of fragments under the 128-register budget of
       // four waves per SIMD (a spill would also put scratch loads into the memory counter and break the
-      // counts below); the other three waves of the SIMD cover the LDS latency instead
+      // counts below); the other three waves of the SIMD cover the LDS latency instead.  (Workgroups of 2 or 4
+      // waves are alone on their SIMD and have the registers: they take the other path.)
       v4i af[MT];
 #pragma unroll
       for (int ss = 0; ss < 4; ++ss) {
