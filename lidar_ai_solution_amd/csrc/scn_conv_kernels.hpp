@@ -394,7 +394,8 @@ struct Mma32<1> {
 // Waves per SIMD the kernel is compiled for: two 8-wave workgroups per CU (128 registers), or one of
 // 9 .. 12 waves.  The 64-channel kernels with 64- and 128-byte input rows take three 8-wave workgroups per
 // CU instead (80 registers without spilling, with a two-stage index ring and one set of A fragments): a
-// lidar frame's 64-channel stage is more tiles than two workgroups per CU hold in one round.
+// lidar frame's 64-channel stage is more tiles than two workgroups per CU hold in one round.  Workgroups of
+// 2 or 4 waves (64 and 128 output channels, launches of few rows) are alone on their SIMDs: 256 registers.
 constexpr bool conv_lds_three_groups(int chunks, int mt, int waves) {
   return mt == 2 && waves == 8 && (chunks == 4 || chunks == 8);
 }
@@ -404,10 +405,10 @@ constexpr int conv_lds_min_waves(int chunks, int mt, int waves) {
 
 // AHEAD = iterations between the issue of an iteration's gathers / weight slab and their use.  1: one stage per
 // wave and two slab buffers, which is what fits the LDS of full CUs, and the only value the dispatch below
-// instantiates.  2: three of each, meant for launches of few rows (at most four 32-row tiles per CU), where
-// nothing competes for the CU and an iteration lasts as long as the round trip of its gathers (about 1 us
-// whatever the layer's width).  NOT DISPATCHED: its first run on the GPU ended in a memory fault whose cause
-// has not been found by reading the code and its assembly; it must not be instantiated before it is.
+// instantiates.  2: three of each, meant for launches of few rows (at most four 32-row tiles per CU).
+// NOT DISPATCHED: its first run on the GPU ended in a memory fault whose cause has not been found by reading
+// the code and its assembly; it must not be instantiated before it is.  (Later measurements with loads issued
+// earlier in the one-stage schedule found that neither gathers nor slabs are late, so it may not pay either.)
 template <int EL, int CHUNKS, int MT, int WAVES, int AHEAD = 1>
 __global__ __launch_bounds__(64 * WAVES, AHEAD > 1 ? 2 : conv_lds_min_waves(CHUNKS, MT, WAVES)) void k_conv_lds(const ConvArgs a) {
   using Acc = typename Mma32<EL>::Acc;
