@@ -15,7 +15,7 @@ from oracle import scn_oracle as O
 pytestmark = pytest.mark.gpu
 
 from tests.gpu_helpers import DEV, GpuRulebook, to_dev  # noqa: E402
-from tests.test_gpu_engine import (FP16_COS, FP16_REL, GRID_XYZ, GRID_ZYX, _compare_dense, _fp16_region_override,  # noqa: E402
+from tests.test_gpu_engine import (FP16_COS, FP16_REL, GRID_XYZ, GRID_ZYX, _compare_dense, _fp16_region_override, _oracle_walk_rebased,  # noqa: E402
                                    _oracle_calibration, _run_engine, note)
 from tests.test_gpu_stages import STAGES, _check_pairs  # noqa: E402
 
@@ -67,8 +67,7 @@ def test_config3_int8_backbone_full_size_and_row_order_invariance(frame250k):
     graphs.apply_int8_plan(g8, tags8, amax, "centerpoint")
     keep = Engine.from_graph(g8, "int8", keep_all=True)
     _run_engine(keep, f, i, GRID_ZYX)
-    rec = {}
-    O.run_graph(g8, f, i, GRID_ZYX, "int8", rec, override=_fp16_region_override(g8, keep))
+    rec = _oracle_walk_rebased(g8, keep, f, i, GRID_ZYX)
     want = rec[g8.nodes[-1].name]["out"]
     # every int8 conv's accumulators at full size
     import ctypes as C
@@ -144,8 +143,7 @@ def test_config5_bevfusion_int8_end_to_end():
     graphs.apply_int8_plan(g8, tags8, amax, "bevfusion")
     keep = Engine.from_graph(g8, "int8", keep_all=True)
     _run_engine(keep, rf, ri, GRID_XYZ)
-    rec = {}
-    O.run_graph(g8, rf, ri, GRID_XYZ, "int8", rec, override=_fp16_region_override(g8, keep))
+    rec = _oracle_walk_rebased(g8, keep, rf, ri, GRID_XYZ)
     want = rec[g8.nodes[-1].name]["out"]
     vox = Voxelization(synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, max_voxels=160000, max_points=300000)
     scn = LidarSCN(g8, vox, order="xyz", precision="int8")

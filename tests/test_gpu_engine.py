@@ -135,8 +135,7 @@ def test_int8_backbone_every_layer_bit_exact(cp_models, centerpoint_input):
     eng = Engine.from_graph(g8, "int8", keep_all=True)
     _run_engine(eng, feats, idx, GRID_ZYX)
     # oracle walk with the engine's fp16-region outputs substituted (see docstring)
-    rec = {}
-    O.run_graph(g8, feats, idx, GRID_ZYX, "int8", rec, override=_fp16_region_override(g8, eng))
+    rec = _oracle_walk_rebased(g8, eng, feats, idx, GRID_ZYX)
     nacc, nout = _check_every_layer(g8, eng, rec)
     print(f"bit-exact: {nacc} int32 accumulator tensors, {nout} int8 tensors")
     assert nacc >= 17 and nout >= 25
@@ -239,6 +238,34 @@ def _fp16_region_override(graph, eng):
     return out
 
 
+def _oracle_walk_rebased(graph, eng, feats, idx, grid):
+    """The oracle's per-node record for an int8 plan that keeps some convolutions in fp16.  Those nodes are
+    first compared with the oracle's own, un-substituted walk at the fp16 tolerance (a stored int8 tensor:
+    codes at most one apart, in under 2 % of the elements); then the walk is repeated with the device's
+    results of exactly those nodes substituted, so that every other tensor can be compared bit for bit."""
+    plain = {}
+    O.run_graph(graph, feats, idx, grid, "int8", plain)
+    ov = _fp16_region_override(graph, eng)
+    for n in graph.nodes:
+        if n.outputs[0] not in ov:
+            continue
+        want = plain[n.name]["out"]
+        got = ov[n.outputs[0]][:, :want.shape[1]]
+        assert got.shape == want.shape and got.dtype == want.dtype, n.name
+        if want.dtype == np.int8:
+            d = np.abs(got.astype(np.int32) - want.astype(np.int32))
+            print(f"fp16-computed {n.name} (int8 store): {np.mean(d != 0):.2e} of the codes differ, max {d.max()}")
+            assert d.max() <= 1 and np.mean(d != 0) < 0.02, n.name
+        else:
+            g, w = got.astype(np.float32), want.astype(np.float32)
+            err = float(np.abs(g - w).max())
+            print(f"fp16-computed {n.name}: max-abs {err:.3e} (ref max {np.abs(w).max():.3e})")
+            assert err <= FP16_REL * max(float(np.abs(w).max()), 1e-6), n.name
+    rec = {}
+    O.run_graph(graph, feats, idx, grid, "int8", rec, override=ov)
+    return rec
+
+
 def test_bevfusion_int8_graph_xyz(bevfusion_input):
     feats, idx = bevfusion_input
     note("BEVFusion-shaped xyz backbone on the 17,748-voxel fixture: fp16 tolerance, int8 bit-exact")
@@ -255,8 +282,7 @@ def test_bevfusion_int8_graph_xyz(bevfusion_input):
     graphs.apply_int8_plan(g8, tags8, amax, "bevfusion")
     keep = Engine.from_graph(g8, "int8", keep_all=True)
     _run_engine(keep, feats, idx, GRID_XYZ)
-    rec = {}
-    O.run_graph(g8, feats, idx, GRID_XYZ, "int8", rec, override=_fp16_region_override(g8, keep))
+    rec = _oracle_walk_rebased(g8, keep, feats, idx, GRID_XYZ)
     nacc, nout = _check_every_layer(g8, keep, rec)
     assert nacc >= 19
     fused = Engine.from_graph(g8, "int8")
