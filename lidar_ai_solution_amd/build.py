@@ -37,8 +37,18 @@ def _run(cmd, verbose):
         print(out)
 
 
-def build(verbose: bool = False, jobs: int = 0) -> str:
-    """Compiles every source to an object file (side by side, `jobs` at a time) and links the library."""
+def _stale(obj: str, src: str) -> bool:
+    """True when obj is older than its source or than any header of csrc/ and include/."""
+    if not os.path.exists(obj):
+        return True
+    t = os.path.getmtime(obj)
+    deps = [src] + glob.glob(os.path.join(HERE, "csrc", "*.hpp")) + glob.glob(os.path.join(ROOT, "include", "*.h"))
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def build(verbose: bool = False, jobs: int = 0, incremental: bool = False) -> str:
+    """Compiles every source to an object file (side by side, `jobs` at a time) and links the library.
+    incremental: keep the object files that are newer than their source and every header."""
     from concurrent.futures import ThreadPoolExecutor
 
     os.makedirs(LIB_DIR, exist_ok=True)
@@ -51,6 +61,8 @@ def build(verbose: bool = False, jobs: int = 0) -> str:
     for src in sources():
         obj = os.path.join(obj_dir, os.path.basename(src) + ".o")
         objs.append(obj)
+        if incremental and not _stale(obj, src):
+            continue
         cmds.append(["hipcc", *compile_flags, "-I" + os.path.join(ROOT, "include"), "-c", src, "-o", obj])
     with ThreadPoolExecutor(max_workers=jobs_) as pool:
         list(pool.map(lambda c: _run(c, verbose), cmds))
@@ -60,5 +72,5 @@ def build(verbose: bool = False, jobs: int = 0) -> str:
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, incremental="--incremental" in sys.argv))
     sys.exit(0)
