@@ -98,6 +98,8 @@ _SIGNATURES = {
     "scn_scatter_dense": (C.c_int, [vp, C.c_int, C.c_float, u32, u32, vp, u32, vp, i5, vp, vp, vp]),
     "scn_scatter_dense_map_cells": (C.c_size_t, [i5, vp]),
     "scn_scatter_dense_with_map": (C.c_int, [vp, C.c_int, C.c_float, u32, u32, vp, u32, vp, i5, vp, vp, vp, vp]),
+    "scn_scatter_dense_noalloc_max_cells": (C.c_size_t, []),
+    "scn_scatter_dense_noalloc": (C.c_int, [vp, C.c_int, C.c_float, u32, u32, vp, u32, vp, i5, vp, vp, vp]),
     "scn_builder_create": (vp, []),
     "scn_builder_destroy": (None, [vp]),
     "scn_builder_push_input": (C.c_int, [vp, C.c_char_p]),

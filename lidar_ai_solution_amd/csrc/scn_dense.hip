@@ -1,5 +1,6 @@
 // Elementwise glue (quantise / dequantise / pad, add + relu) and sparse -> dense of the SCN path (gfx950).
 #include "scn_device.hpp"
+#include <mutex>
 
 #include <algorithm>
 #include <cstdlib>
@@ -367,6 +368,38 @@ int permute_dense(const void* in, const int64_t in_shape[5], const int perm[5], 
 
 using namespace scn;
 
+// ---------------------------------------------------------------- allocation-free sparse -> dense
+// scn_scatter_dense_with_map with the row map in a static device array instead of a caller's workspace: for
+// callers that cannot allocate (HIP graph capture, serving loops, harnesses that forbid hipMalloc).  The array
+// exists once per GPU for the life of the process; its device address is looked up once per device, with that
+// device current, and only that address -- never the array's name, which in host code is a stand-in and not a
+// device address -- is passed to kernels.  Every call on a GPU uses that GPU's one array, so calls that overlap
+// on one GPU (two streams, two threads) race; the map is cleared by a fill kernel at the start of every call.
+#define SCN_NOALLOC_MAX_CELLS (1u << 18)
+static __device__ __align__(256) int32_t scratch[SCN_NOALLOC_MAX_CELLS];
+
+namespace {
+constexpr int kMaxDevices = 64;
+int32_t* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+int scratch_of_current_device(int32_t** out) {
+  int dev = -1;
+  SCN_HIP(hipGetDevice(&dev));
+  SCN_REQUIRE(dev >= 0 && dev < kMaxDevices, SCN_ERR_UNSUPPORTED, "device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    SCN_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    SCN_REQUIRE(p != nullptr, SCN_ERR_HIP, "hipGetSymbolAddress returned a null address");
+    g_scratch_ptr[dev] = static_cast<int32_t*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return SCN_OK;
+}
+}  // namespace
+
+
 extern "C" {
 // ---- elementwise / dense --------------------------------------------------------------------
 int scn_convert_rows(const void* in_dev, int in_dtype, uint32_t in_c, uint32_t in_ld, float in_range, void* out_dev,
@@ -397,6 +430,27 @@ int scn_scatter_dense_with_map(const void* feat_dev, int dtype, float dynamic_ra
                                const int perm[5], void* out_fp16_dev, int32_t* cell_map_dev, void* stream) {
   return scatter_dense(feat_dev, dtype, dynamic_range, c, ld, indices_dev, n, n_dev, dense_shape, perm, out_fp16_dev,
                        (hipStream_t)stream, false, cell_map_dev, false);
+}
+
+
+size_t scn_scatter_dense_noalloc_max_cells(void) { return SCN_NOALLOC_MAX_CELLS; }
+
+int scn_scatter_dense_noalloc(const void* feat_dev, int dtype, float dynamic_range, uint32_t c, uint32_t ld,
+                              const int32_t* indices_dev, uint32_t n, const uint32_t* n_dev, const int dense_shape[5],
+                              const int perm[5], void* out_fp16_dev, void* stream) {
+  SCN_REQUIRE(dense_shape, SCN_ERR_INVALID, "scatter_dense: null pointer");
+  const size_t cells = scatter_dense_map_cells(dense_shape, perm);
+  SCN_REQUIRE(cells != 0, SCN_ERR_UNSUPPORTED,
+              "scn_scatter_dense_noalloc: the layout takes no row map (channel axis must be outermost after the "
+              "Transpose and D0*D1*D2 a multiple of 8)");
+  SCN_REQUIRE(cells <= SCN_NOALLOC_MAX_CELLS, SCN_ERR_CAPACITY,
+              "scn_scatter_dense_noalloc: D0*D1*D2 = %zu cells exceed the static row map of %u cells", cells,
+              (unsigned)SCN_NOALLOC_MAX_CELLS);
+  int32_t* map = nullptr;
+  int rc = scratch_of_current_device(&map);
+  if (rc) return rc;
+  return scatter_dense(feat_dev, dtype, dynamic_range, c, ld, indices_dev, n, n_dev, dense_shape, perm, out_fp16_dev,
+                       (hipStream_t)stream, false, map, false);
 }
 
 }  // extern "C"
