@@ -35,9 +35,6 @@ inline bool check_hip_api_(hipError_t e, const char* call, int line, const char*
     __VA_ARGS__;                                                                    \
     spconv::check_hip_api_(hipPeekAtLastError(), #__VA_ARGS__, __LINE__, __FILE__); \
   } while (0)
-// spelling of the reference, for sources that have not been renamed yet
-#define check_cuda_api(call) check_hip_api(call)
-#define check_cuda_kernel(...) check_hip_kernel(__VA_ARGS__)
 
 #define spconv_assertf(cond, fmt, ...)                                                                        \
   do {                                                                                                        \

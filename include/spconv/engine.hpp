@@ -6,8 +6,8 @@
 // compiling after its CUDA runtime calls are turned into HIP ones; `void* stream` is a hipStream_t.
 //
 // Differences that a caller can observe:
-//   * build()'s sortmask / enable_blackwell / with_auxiliary_stream are accepted and ignored
-//     (performance-only switches of the reference).
+//   * build()'s enable_blackwell is accepted and ignored; sortmask and with_auxiliary_stream are passed on
+//     (performance-only switches: results are bit-identical with and without them).
 //   * device buffers are allocated when the grid size is set (set_grid_size) so that forward() is
 //     legal inside hipStreamBeginCapture from the very first call.
 #ifndef SCN_SPCONV_ENGINE_HPP

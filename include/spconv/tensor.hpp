@@ -10,6 +10,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include "../scn_c_api.h"
+
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -208,7 +210,8 @@ struct Tensor {
   void to_host_(void* stream = nullptr) { *this = to_host(stream); }
   void memset(unsigned char value = 0, void* stream = nullptr) {
     if (!bytes()) return;
-    if (device()) (void)hipMemsetAsync(ptr(), value, bytes(), (hipStream_t)stream); else std::memset(ptr(), value, bytes());
+    // device memory is filled by a kernel of the library: a memset node must not end up in a captured graph
+    if (device()) (void)scn_memset_async(ptr(), value, bytes(), stream); else std::memset(ptr(), value, bytes());
   }
   // fills an Int32 tensor with 0..num-1
   void arange(size_t num, void* stream = nullptr) {

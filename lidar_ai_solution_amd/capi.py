@@ -64,6 +64,7 @@ _SIGNATURES = {
     "scn_get_log_level": (C.c_int, []),
     "scn_set_log_callback": (None, [LOG_CALLBACK, vp]),
     "scn_log": (None, [C.c_char_p, C.c_int, C.c_int, C.c_char_p]),
+    "scn_memset_async": (C.c_int, [vp, C.c_ubyte, C.c_size_t, vp]),
     "scn_hash_u64": (C.c_uint64, [C.c_uint64]),
     "scn_hash_capacity_for": (C.c_size_t, [u32]),
     "scn_hash_build": (C.c_int, [vp, C.c_size_t, vp, u32, vp, i3, vp]),

@@ -61,6 +61,21 @@ int fill_multi(const FillJob* jobs, int n_jobs, uint32_t* count_dst, const uint3
   return SCN_OK;
 }
 
+// Byte fill of an arbitrary range: the 16-byte aligned body in whole vectors, head and tail byte by byte.
+__global__ __launch_bounds__(256) void k_fill_bytes(unsigned char* __restrict__ p, unsigned char value, size_t bytes) {
+  const size_t head = min(bytes, (size_t)((16 - ((uintptr_t)p & 15)) & 15));
+  const size_t body = (bytes - head) / 16;
+  const size_t stride = (size_t)gridDim.x * 256;
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const uint32_t v = value * 0x01010101u;
+  const uint4 v4 = make_uint4(v, v, v, v);
+  uint4* b = reinterpret_cast<uint4*>(p + head);
+  for (size_t k = i; k < body; k += stride) b[k] = v4;
+  if (i < head) p[i] = value;
+  const size_t tail0 = head + body * 16;
+  if (tail0 + i < bytes && i < 16) p[tail0 + i] = value;
+}
+
 int fill_u32(void* p, uint32_t value, size_t count, hipStream_t stream) {
   if (count == 0) return SCN_OK;
   SCN_REQUIRE(((uintptr_t)p & 15) == 0, SCN_ERR_INVALID, "fill_u32: pointer not 16-byte aligned");
@@ -825,6 +840,17 @@ __global__ __launch_bounds__(256) void k_vox_mean(const _Float16* __restrict__ p
 using namespace scn;
 
 extern "C" {
+
+int scn_memset_async(void* dev, unsigned char value, size_t bytes, void* stream) {
+  if (bytes == 0) return SCN_OK;
+  SCN_REQUIRE(dev, SCN_ERR_INVALID, "scn_memset_async: null pointer");
+  size_t blocks = (bytes / 16 + 255) / 256;
+  blocks = blocks < 1 ? 1 : blocks > 4096 ? 4096 : blocks;
+  hipLaunchKernelGGL(k_fill_bytes, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (unsigned char*)dev, value,
+                     bytes);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
 
 uint64_t scn_hash_u64(uint64_t key) { return hash64(key); }
 size_t scn_hash_capacity_for(uint32_t n) { return hash_capacity_for(n); }

@@ -523,9 +523,7 @@ static bool build_engine(scn_engine& e) {
         }
         // output tensor + fusion of a following Add (+Relu) / Relu
         int t_out = n.out;
-        st.relu = n.activation == "ReLU" ? 1 : 0;
-        if (!n.activation.empty() && n.activation != "ReLU" && n.activation != "None")
-          SCN_LOGW("node %s: activation '%s' is not supported and is ignored", n.name.c_str(), n.activation.c_str());
+        st.relu = n.activation == "ReLU" ? 1 : 0;   // (anything but ReLU / None was refused by push_sparse_conv)
         int out_dtype = (plan.outp[i] == SCN_PRECISION_INT8 && plan.range[n.out] > 0.f) ? SCN_DTYPE_INT8 : SCN_DTYPE_FP16;
         float out_range = out_dtype == SCN_DTYPE_INT8 ? plan.range[n.out] : 0.f;
         if (plan.outp[i] == SCN_PRECISION_INT8 && out_dtype != SCN_DTYPE_INT8)
@@ -1233,6 +1231,14 @@ int scn_builder_push_sparse_conv(scn_builder* b, const char* name, int x, const 
   (void)fixed_launch_points;  // launch sizes always come from host-side bounds; nothing to fix
   if (!b || !b->valid_tensor(x) || !weight || !weight_shape || !kernel_size) {
     set_error("push_sparse_conv(%s): invalid arguments", name ? name : "");
+    return -1;
+  }
+  // What cannot be computed is refused when it is pushed, so that the builder and the loader return nullptr
+  // instead of an engine with different arithmetic (the loader's contract for a model it cannot run,
+  // libraries/3DSparseConvolution/src/onnx-parser.cpp:216-219).  The exporters can write other activations
+  // (CUDA-CenterPoint/qat/onnx_export/exptool.py:167-172).
+  if (activation && *activation && strcmp(activation, "ReLU") != 0 && strcmp(activation, "None") != 0) {
+    set_error("push_sparse_conv(%s): activation '%s' is not supported (ReLU or None)", name ? name : "", activation);
     return -1;
   }
   if (inverse && (submanifold || !rulebook || !*rulebook)) {

@@ -18,9 +18,10 @@ from .onnx_dialect import Graph, Node
 
 
 class _Builder:
-    def __init__(self, seed: int, weight_std: float = 0.02):
+    def __init__(self, seed: int, weight_std: float = 0.02, output_bound: int = 200000):
         self.rng = np.random.default_rng(seed)
         self.std = weight_std
+        self.output_bound = int(output_bound)
         self.nodes: List[Node] = []
         self.inits: Dict[str, np.ndarray] = {}
         self.next_tensor = 1
@@ -45,7 +46,7 @@ class _Builder:
         self.nodes.append(Node("SparseConvolution", f"conv{i}", [x, f"spconv{i}.weight", f"spconv{i}.bias"], [y], {
             "ndim": 3, "in_channels": cin, "out_channels": cout,
             "kernel_size": list(ksize), "stride": list(stride), "padding": list(padding), "dilation": [1, 1, 1],
-            "output_bound": 200000, "transposed": 0, "inverse": int(inverse), "groups": 1,
+            "output_bound": self.output_bound, "transposed": 0, "inverse": int(inverse), "groups": 1,
             "subm": int(subm), "rulebook": rulebook, "activation": activation, "tag": tag,
         }))
         return y
@@ -79,13 +80,15 @@ def _strip_tags(nodes: List[Node]) -> Dict[str, str]:
 
 
 def centerpoint_scn(seed: int = 0, in_channels: int = 5, grid_zyx: Sequence[int] = (41, 1440, 1440),
-                    channels: Sequence[int] = (16, 32, 64, 128), weight_std: float = 0.02
-                    ) -> Tuple[Graph, Dict[str, str]]:
+                    channels: Sequence[int] = (16, 32, 64, 128), weight_std: float = 0.02,
+                    output_bound: int = 200000) -> Tuple[Graph, Dict[str, str]]:
     """CenterPoint `SpMiddleResNetFHD`-shaped graph, zyx index order, all fp16.
 
+    output_bound is the row capacity every convolution carries (the exporter's `output_bound` attribute,
+    CUDA-CenterPoint/qat/onnx_export/exptool.py:178-205); the random weights do not depend on it.
     Returns the graph and a map node name -> module path (used by the precision plans).
     """
-    b = _Builder(seed, weight_std)
+    b = _Builder(seed, weight_std, output_bound)
     c0, c1, c2, c3 = channels
     x = b.conv("0", in_channels, c0, (3, 3, 3), subm=True, rulebook="res0", tag="conv_input")
     x = b.block(x, c0, "res0", "conv1.0")
@@ -114,10 +117,10 @@ def centerpoint_scn(seed: int = 0, in_channels: int = 5, grid_zyx: Sequence[int]
 
 
 def bevfusion_scn(seed: int = 0, in_channels: int = 5, grid_xyz: Sequence[int] = (1440, 1440, 41),
-                  channels: Sequence[int] = (16, 32, 64, 128), weight_std: float = 0.02
-                  ) -> Tuple[Graph, Dict[str, str]]:
+                  channels: Sequence[int] = (16, 32, 64, 128), weight_std: float = 0.02,
+                  output_bound: int = 200000) -> Tuple[Graph, Dict[str, str]]:
     """BEVFusion lidar `SparseEncoder`-shaped graph, xyz index order, all fp16."""
-    b = _Builder(seed, weight_std)
+    b = _Builder(seed, weight_std, output_bound)
     c0, c1, c2, c3 = channels
     x = b.conv("0", in_channels, c0, (3, 3, 3), subm=True, rulebook="subm1", tag="conv_input")
     g = list(grid_xyz)

@@ -40,6 +40,27 @@ def test_host_side_argument_checks_need_no_gpu():
         L.scn_set_log_level(1)
 
 
+@pytest.mark.parametrize("activation", ["Sigmoid", "LeakyReLU"])
+def test_model_with_an_unsupported_activation_does_not_load(activation, tmp_path):
+    """The exporters can write activations the engine has no epilogue for
+    (CUDA-CenterPoint/qat/onnx_export/exptool.py:167-172); the loader's contract for a model it cannot run is a
+    null engine (libraries/3DSparseConvolution/src/onnx-parser.cpp:216-219), never an engine that computes
+    something else.  The refusal happens while the node is pushed, before anything touches a GPU."""
+    L = capi.lib()
+    g = graphs.single_subm_layer(seed=3)
+    g.nodes[0].attrs["activation"] = activation
+    path = str(tmp_path / "act.scn.onnx")
+    onnx_dialect.save(g, path)
+    L.scn_set_log_level(99)
+    try:
+        for precision in (capi.PRECISION_FP16, capi.PRECISION_INT8):
+            assert not L.scn_engine_create_from_onnx(path.encode(), precision, 0, 10000, None)
+            msg = L.scn_last_error()
+            assert activation.encode() in msg and b"not supported" in msg
+    finally:
+        L.scn_set_log_level(1)
+
+
 def test_log_callback_receives_messages():
     L = capi.lib()
     seen = []
@@ -110,3 +131,30 @@ def test_tensor_file_round_trip(tmp_path, centerpoint_input):
     ref = "/root/reference/libraries/3DSparseConvolution/workspace/centerpoint/in_features.torch.fp16.tensor"
     if os.path.exists(ref):  # the reference's own file parses to the committed fixture
         assert np.array_equal(tensor.load(ref).view(np.uint16), feats.view(np.uint16))
+
+
+def test_compare_report_numbers_and_row_order_invariance(tmp_path, capsys):
+    """The agreement report of the reference's tool/compare.py:71-118: its numbers on a hand-made case, and that
+    a sparse tensor compares equal to a row permutation of itself once rows are put into coordinate order."""
+    from lidar_ai_solution_amd import compare
+    a = np.array([[0.0, 1.0, 2.0, 3.0], [4.0, 5.0, 6.0, 7.0]], np.float16)
+    b = a.copy()
+    b[0, 1] += 1.0      # differences: 1.0, 0.5, 0.25 and five zeros
+    b[1, 0] += 0.5
+    b[1, 3] += 0.25
+    m = compare.metrics(a, b)
+    assert m["absdiff_max"] == 1.0 and m["absdiff_sum"] == 1.75 and m["numel"] == 8
+    assert (m["above_75pct_of_max"], m["above_50pct_of_max"], m["above_25pct_of_max"], m["differ"], m["equal"]) == (1, 1, 2, 3, 5)
+    x, y = a.astype(np.float64).ravel(), b.astype(np.float64).ravel()
+    assert abs(m["cosine"] - x @ y / np.sqrt((x @ x) * (y @ y))) < 1e-12
+    rng = np.random.default_rng(0)
+    idx = np.stack([np.zeros(50, np.int32), rng.integers(0, 5, 50), rng.integers(0, 9, 50), np.arange(50)], 1).astype(np.int32)
+    feat = rng.standard_normal((50, 8)).astype(np.float16)
+    perm = rng.permutation(50)
+    for name, f, i in (("p", feat, idx), ("q", feat[perm], idx[perm])):
+        tensor.save(f, str(tmp_path / f"{name}.f.tensor"))
+        tensor.save(i, str(tmp_path / f"{name}.i.tensor"))
+    assert compare.main([str(tmp_path / "p.f.tensor:p.i.tensor"), str(tmp_path / "q.f.tensor:q.i.tensor"),
+                         "--dense-grid", "5x9x50", "--detail"]) == 0
+    out = capsys.readouterr().out
+    assert "[absdiff]: max:0.0" in out and "[absdiff = 0]: 100.000 %, 400" in out and "[cosine]: 100.000 %" in out

@@ -457,6 +457,89 @@ def test_cpp_example_driver_matches_python_engine(cp_models, centerpoint_input, 
         assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
 
 
+def _example(name):
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "lidar_ai_solution_amd", "examples", name)
+    if not os.path.exists(exe):
+        pytest.skip("example driver not built (python -c 'import __graft_entry__ as g; g.build()')")
+    return exe
+
+
+def _cp_model_files(cp_models, centerpoint_input, tmp_path, rows=None):
+    from lidar_ai_solution_amd import tensor
+    feats, idx = centerpoint_input
+    if rows:
+        feats, idx = feats[:rows], idx[:rows]
+    model = str(tmp_path / "cp.int8.scn.onnx")
+    onnx_dialect.save(cp_models[1], model)
+    tensor.save(feats, str(tmp_path / "f.tensor"))
+    tensor.save(idx, str(tmp_path / "i.tensor"))
+    return [model, str(tmp_path / "f.tensor"), str(tmp_path / "i.tensor"), "41", "1440", "1440", "int8", str(tmp_path / "out")]
+
+
+@pytest.mark.parametrize("mode", [{}, {"SCN_USE_DDS": "1"}, {"SCN_USE_HIPGRAPH": "1"},
+                                  {"SCN_USE_HIPGRAPH": "1", "SCN_AUX_STREAM": "1", "SCN_SORTMASK": "1"}])
+def test_cpp_stress_shrinking_inputs(mode, cp_models, centerpoint_input, tmp_path):
+    """The reference driver's --stress (libspconv/example/infer.cpp:344-367): the input loses a seeded random
+    number of rows (0..199) before every forward, through the device-side count when a graph or DDS is in use,
+    by re-referencing the input tensors otherwise.  Here every forward is also compared, bit for bit, with a
+    plain second engine run on the same rows; the driver stops at the first mismatch."""
+    import subprocess
+    exe = _example("infer")
+    args = _cp_model_files(cp_models, centerpoint_input, tmp_path)
+    note(f"C++ stress, 60 forwards, switches {mode}")
+    env = dict(os.environ, STRESS="60", SCN_SEED="11", **mode)
+    r = subprocess.run([exe] + args, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=170)
+    print(r.stdout)
+    assert r.returncode == 0 and "Stress test passed" in r.stdout, r.stdout
+
+
+def test_cpp_search_best_perf_lists_every_configuration(cp_models, centerpoint_input, tmp_path):
+    """The reference driver's --search_best_perf (src/infer.cpp:371-466): 100 + 1000 timed forwards per
+    combination of {graph with three launch bounds, direct} x sortmask x auxiliary stream, sorted by latency."""
+    import subprocess
+    exe = _example("infer")
+    args = _cp_model_files(cp_models, centerpoint_input, tmp_path, rows=20000)
+    note("C++ search_best_perf on the first 20,000 rows of the fixture: 16 configurations")
+    env = dict(os.environ, SEARCH_BEST_PERF="1")
+    r = subprocess.run([exe] + args, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=170)
+    print(r.stdout)
+    assert r.returncode == 0, r.stdout
+    assert "Best configuration found" in r.stdout and "Sorted configuration list (16 configurations)" in r.stdout
+    lat = [float(l.rsplit("Latency:", 1)[1].split("ms")[0]) for l in r.stdout.splitlines() if l.strip()[:3].rstrip(".").isdigit()]
+    assert len(lat) == 16 and lat == sorted(lat) and 0.0 < lat[0] < 50.0
+
+
+@pytest.mark.parametrize("aux", [False, True])
+def test_cpp_lidar_scn_glue_one_graph_for_voxelization_and_backbone(aux, nuscenes_frame, tmp_path):
+    """bevfusion::lidar::SCN (include/bevfusion/lidar-scn.hpp; the reference's lidar-scn.cpp:34-50) from C++:
+    points -> BEV equals the Python glue's bits, and one HIP graph holding voxelization + backbone replays
+    bit-exactly on frames of 1, 1/2 and 1/3 of the points (checked inside the example against eager forwards)."""
+    import subprocess
+    from lidar_ai_solution_amd import tensor
+    exe = _example("lidar_scn")
+    pts = nuscenes_frame
+    g16, tags = graphs.bevfusion_scn(seed=5)
+    rf, ri, _ = O.voxelize(pts, synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, order="xyz")
+    amax = _oracle_calibration(g16, rf, ri, GRID_XYZ)
+    g8, tags8 = graphs.bevfusion_scn(seed=5)
+    graphs.apply_int8_plan(g8, tags8, amax, "bevfusion")
+    model = str(tmp_path / "bev.int8.scn.onnx")
+    onnx_dialect.save(g8, model)
+    tensor.save(pts, str(tmp_path / "points.tensor"))
+    note(f"C++ lidar glue: {pts.shape[0]} points -> BEV, auxiliary stream {aux}")
+    prefix = str(tmp_path / "bev")
+    r = subprocess.run([exe, model, str(tmp_path / "points.tensor"), "xyz", "int8", prefix] + (["aux"] if aux else []),
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=170)
+    print(r.stdout)
+    assert r.returncode == 0 and r.stdout.count("bit-exact") == 4, r.stdout
+    got = tensor.load(prefix + ".eager.tensor")
+    vox = Voxelization(synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, max_voxels=160000, max_points=300000)
+    scn = LidarSCN(g8, vox, order="xyz", precision="int8")
+    want = scn.forward(to_dev(pts)).torch().cpu().numpy()
+    assert got.shape == want.shape == (1, 256, 180, 180)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16)) and np.count_nonzero(got) > 100000
+
+
 def test_legacy_single_call_interface_and_precision_overrides(cp_models, centerpoint_input, tmp_path):
     """The older engine interface (forward(shapes, types, pointers, ...) -> DTensor*, set_node_precision_by*,
     reconfigure) through the C++ caller built against include/legacy/spconv/engine.hpp, and the loader's

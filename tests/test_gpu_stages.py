@@ -517,6 +517,36 @@ def test_scatter_dense_with_row_map():
                 assert np.array_equal(out.cpu().numpy().view(np.uint16), ref.view(np.uint16))
 
 
+def test_memset_kernel_any_alignment_and_inside_a_graph():
+    """scn_memset_async (Tensor::memset of the C++ header): byte ranges with unaligned heads and tails, and
+    recorded into a HIP graph that is replayed with other work in between."""
+    L = capi.lib()
+    note("byte fill kernel: unaligned ranges, then graph replays")
+    buf = torch.zeros(100003, dtype=torch.uint8, device=DEV)
+    for off, n, v in ((0, 100003, 7), (1, 15, 9), (3, 4096 + 5, 250), (16, 64, 1), (17, 1, 33), (5, 0, 99)):
+        buf.fill_(0)
+        capi.check(L.scn_memset_async(C.c_void_p(buf.data_ptr() + off), v, n, stream()))
+        torch.cuda.synchronize()
+        want = np.zeros(100003, np.uint8)
+        want[off:off + n] = v
+        assert np.array_equal(buf.cpu().numpy(), want), (off, n, v)
+    st = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(st):
+        capi.check(L.scn_memset_async(C.c_void_p(buf.data_ptr() + 2), 5, 1001, C.c_void_p(st.cuda_stream)))
+    torch.cuda.synchronize()
+    with torch.cuda.graph(g, stream=st):
+        capi.check(L.scn_memset_async(C.c_void_p(buf.data_ptr() + 2), 5, 1001, C.c_void_p(st.cuda_stream)))
+    for rep in range(3):
+        buf.fill_(rep + 10)
+        assert np.isfinite(torch.randn(1 << 18, device=DEV).sum().item())
+        g.replay()
+        torch.cuda.synchronize()
+        want = np.full(100003, rep + 10, np.uint8)
+        want[2:1003] = 5
+        assert np.array_equal(buf.cpu().numpy(), want), rep
+
+
 # ----------------------------------------------------------------------------- voxelization
 def _voxelizer(max_voxels=160000, max_points=300000):
     p = capi.VoxelizationParam()
