@@ -55,6 +55,9 @@ def parse_args():
                     help="row capacity of every convolution (the model's output_bound attribute).  The default is above "
                          "every stage of the synthetic frame, so nothing is truncated; 200000 is the exporters' figure, "
                          "at which stage 1 of that frame is cut (a secondary run)")
+    ap.add_argument("--sortmask", dest="sortmask", action="store_true", default=False,
+                    help="the reference loader's sortmask switch: rows of the narrow layers' rulebooks are sorted by "
+                         "their sets of kernel offsets so that a tile visits few offsets (results are identical)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="first launch a plain copy kernel of known size (k_convert_rows fp16->fp16, 512 MiB read + "
                          "512 MiB written, 3 launches): the reference point that scales FETCH_SIZE / WRITE_SIZE counters")
@@ -262,7 +265,7 @@ def main():
         graphs.apply_int8_plan(graph, tags, amax, "centerpoint")
     # with_auxiliary_stream is the reference's load_engine_from_onnx option: rulebooks are built on a second
     # stream ahead of the convolutions (per-step profiling below runs them in line, on one stream)
-    eng = Engine.from_graph(graph, args.precision, with_auxiliary_stream=not args.no_aux_stream)
+    eng = Engine.from_graph(graph, args.precision, with_auxiliary_stream=not args.no_aux_stream, sortmask=args.sortmask)
     eng.set_input(feats, idx, GRID_ZYX)
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
@@ -445,7 +448,7 @@ def main():
                    "active_voxels": int(nvox), "grid": list(GRID_ZYX), "output_bound": args.output_bound,
                    "truncated_by_output_bound": bool(truncated),
                    "launch": "hip graph replay" if use_graph else "direct launches",
-                   "auxiliary_stream": not args.no_aux_stream, "output": out_view.shape},
+                   "auxiliary_stream": not args.no_aux_stream, "sortmask": bool(args.sortmask), "output": out_view.shape},
         "voxels_per_s": round(nvox * 1e3 / ms_per_step, 1),
         "voxelization_ms": round(vox_ms, 4),
         "host_enqueue_ms_per_step": round(enqueue_ms, 4),

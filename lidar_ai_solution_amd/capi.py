@@ -83,6 +83,8 @@ _SIGNATURES = {
     "scn_rulebook_build_subm": (C.c_int, [vp, vp, u32, vp, i3, i3, i3, vp]),
     "scn_rulebook_build_sparse": (C.c_int, [vp, vp, u32, vp, i3, i3, i3, i3, i3, vp]),
     "scn_rulebook_build_inverse": (C.c_int, [vp, vp, vp, vp]),
+    "scn_rulebook_build_plan": (C.c_int, [vp, C.c_int, vp]),
+    "scn_rulebook_plan": (C.c_int, [vp, C.POINTER(vp), C.POINTER(vp), C.POINTER(vp)]),
     "scn_rulebook_nbr": (vp, [vp]),
     "scn_rulebook_nbr_ld": (u32, [vp]),
     "scn_rulebook_out_indices": (vp, [vp]),

@@ -111,8 +111,19 @@ bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* 
   return true;
 }
 
+bool conv_tile_covers(const ConvWeights& w) {
+  static const bool off = [] {
+    const char* e = getenv("SCN_CONV_IMPL");
+    return e && (!strcmp(e, "lds") || !strcmp(e, "rows"));
+  }();
+  if (off || w.kvol > 31 || w.mtiles32 < 1 || w.mtiles32 > 2) return false;
+  if (w.chunks != 1 && w.chunks != 2 && w.chunks != 4) return false;
+  // the whole weight tensor stays in LDS: [steps32][mtiles32] fragments of 1 KB
+  return (size_t)w.steps32 * w.mtiles32 * 1024 + 512 <= 60 * 1024;
+}
+
 int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, const uint32_t* n_out_dev,
-                 uint32_t n_bound, uint32_t n_hint, const scn_conv_io& io, hipStream_t stream) {
+                 uint32_t n_bound, uint32_t n_hint, const scn_conv_io& io, hipStream_t stream, const PlanView* plan) {
   if (n_bound == 0) return SCN_OK;
   const int esz = w.precision == SCN_PRECISION_INT8 ? 1 : 2;
   SCN_REQUIRE(io.x_dev && io.out_dev, SCN_ERR_INVALID, "conv: null input or output");
@@ -142,6 +153,13 @@ int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, cons
   a.n_out_dev = n_out_dev;
   a.n_bound = n_bound;
   a.wfrag = w.wfrag.as<uint4>();
+  a.wfrag32 = w.wfrag32.as<uint4>();
+  a.steps32 = w.steps32;
+  if (plan && plan->tmask && conv_tile_covers(w)) {
+    a.tmask = plan->tmask;
+    a.perm = plan->perm;
+    if (plan->nbr) a.nbr = plan->nbr;
+  }
   a.zrow = w.zrow.as<char>();
   a.steps = w.steps;
   a.wscale = w.wscale.as<float>();
@@ -214,9 +232,17 @@ int scn_conv_forward(const scn_conv* c, const scn_rulebook* rb, const scn_conv_i
   SCN_REQUIRE(rb->rb.built, SCN_ERR_INVALID, "scn_conv_forward: rulebook not built");
   SCN_REQUIRE(rb->rb.geom.kvol == c->w.kvol, SCN_ERR_INVALID, "scn_conv_forward: kernel volume mismatch (%d vs %d)",
               rb->rb.geom.kvol, c->w.kvol);
+  PlanView pv;
+  const TilePlan& tp = rb->rb.plan;
+  if (tp.built) {
+    pv.tmask = tp.tmask.as<uint32_t>();
+    if (tp.sorted) {
+      pv.perm = tp.perm.as<uint32_t>();
+      pv.nbr = tp.nbr.as<int32_t>();
+    }
+  }
   return conv_forward(c->w, rb->rb.nbr.as<int32_t>(), rb->rb.ld, rb->rb.n_out_dev(), rb->rb.n_bound_out,
-                      rb->rb.n_out_hint(), *io,
-                      (hipStream_t)stream);
+                      rb->rb.n_out_hint(), *io, (hipStream_t)stream, tp.built ? &pv : nullptr);
 }
 
 }  // extern "C"

@@ -37,11 +37,27 @@ struct ConvArgs {
   int relu2;
   int out_vec16;     // output rows are 16-byte aligned and a multiple of 16 bytes: 16-byte stores allowed
   const char* zrow;  // 512 bytes of zeros (gather source of lanes without a neighbour), then 256 words of -1
+  // tile plan of the rulebook (k_conv_tile only; see TilePlan): one word per 32-row tile with the kernel offsets
+  // at which some row of the tile has a neighbour, and, when the rows were sorted by their offset sets, the row
+  // that each position of the plan order stands for (nbr is then the table in plan order)
+  const uint32_t* tmask = nullptr;
+  const uint32_t* perm = nullptr;
+  const uint4* wfrag32 = nullptr;  // weights in 32x32 MFMA fragment order, steps32 K-steps
+  int steps32 = 0;
+};
+
+// What a convolution launch may use of a rulebook's tile plan.
+struct PlanView {
+  const uint32_t* tmask = nullptr;
+  const uint32_t* perm = nullptr;   // nullptr: plan order = row order
+  const int32_t* nbr = nullptr;     // table in plan order (sorted plans), else nullptr
 };
 
 // Launch the kernel for these weights (one definition per element type, each in its own translation unit).
 // n_hint: expected number of output rows.  Returns false when no kernel covers the shape.
 bool conv_dispatch_int8(const ConvWeights& w, uint32_t n_hint, ConvArgs& a, hipStream_t stream);
 bool conv_dispatch_fp16(const ConvWeights& w, uint32_t n_hint, ConvArgs& a, hipStream_t stream);
+// Shapes the tile-plan kernel covers (narrow layers: input rows of at most 64 bytes, at most 64 output channels).
+bool conv_tile_covers(const ConvWeights& w);
 
 }  // namespace scn

@@ -867,6 +867,182 @@ __global__ __launch_bounds__(64 * WAVES, AHEAD > 1 ? 2 : conv_lds_min_waves(CHUN
   }
 }
 
+// --------------------------------------------------------------------------------------------
+// Tile-plan kernel for the narrow layers (input rows of 16 .. 64 bytes, at most 64 output channels).
+// In a lidar frame's first stages a row has 2 .. 10 of its 27 neighbours, so what such a layer costs is not
+// arithmetic but the slots it visits: this kernel visits, per 32-row tile, only the kernel offsets named in the
+// tile's mask (see TilePlan), and with a sorted plan the rows of a tile share most of theirs.
+//   * persistent workgroups of 8 waves: the whole weight tensor (14 .. 56 KB) is copied to LDS once, after that
+//     the waves never synchronise again; wave w of workgroup g takes tiles 8 g + w, + 8 * gridDim.x, ...
+//   * a wave's step: up to UNR offsets of the mask -> their table entries (one coalesced 128-byte load per
+//     offset) -> the neighbour rows straight into the B operand (16 bytes per lane; rows of 16 bytes pair two
+//     offsets in one MFMA, K-half = offset) -> A fragments from LDS -> MFMA.  No LDS staging of rows: with one
+//     16-byte chunk per lane there is nothing to coalesce.
+//   * positions of a sorted plan are not rows: the epilogue stores (and reads the residual of) row perm[pos].
+// Results are bit-identical to the other kernels: a row's products are added in offset order, integers exactly,
+// fp16 products in fp32 with zero terms left out.
+template <int EL, int CHUNKS, int MT>
+__global__ __launch_bounds__(512, 4) void k_conv_tile(const ConvArgs a) {
+  using Acc = typename Mma32<EL>::Acc;
+  using Acc4 = typename Mma32<EL>::Acc4;
+  constexpr int WAVES = 8;
+  constexpr int KS = CHUNKS >= 2 ? CHUNKS / 2 : 1;   // MFMAs per offset and output tile (16-byte rows: half of one)
+  constexpr int UNR = CHUNKS >= 4 ? 2 : 4;           // offsets (16-byte rows: offset pairs) in flight per step
+  extern __shared__ v4i wl[];                        // [steps32][MT][64] A fragments, then bias[MT*32], scale[MT*32]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, ln = lane & 31, lh = lane >> 5;
+  const int nfrag = a.steps32 * MT * 64;
+  {
+    const v4i* __restrict__ src = reinterpret_cast<const v4i*>(a.wfrag32);
+    for (int i = tid; i < nfrag; i += 64 * WAVES) wl[i] = src[i];
+  }
+  float* ep = reinterpret_cast<float*>(wl + nfrag);
+  const int cout_pad = (a.cout + 15) & ~15;
+  if (tid < MT * 32) {
+    const bool okc = tid < cout_pad;
+    ep[tid] = okc ? a.bias[tid] : 0.f;
+    ep[MT * 32 + tid] = (EL == 0 && okc) ? a.x_scale * a.wscale[tid] : 0.f;
+  }
+  __syncthreads();
+
+  const uint32_t n = eff_n(a.n_out_dev, a.n_bound);
+  const uint32_t tiles = (n + 31u) >> 5;
+  const uint32_t ldb = a.x_ld_bytes;
+  const char* __restrict__ xb = a.x;
+  const char* __restrict__ zrow = a.zrow;
+  const bool out8 = a.out_dtype == SCN_DTYPE_INT8;
+  int mode = 0;
+  if (!a.acc) {
+    if (!a.res)
+      mode = out8 ? 1 : 2;
+    else if (a.res_dtype == a.out_dtype && a.mid_dtype == a.out_dtype && (out8 || (a.a_rq_r <= 0.f && a.b_rq_r <= 0.f)))
+      mode = out8 ? 3 : 4;
+  }
+  const float lo1 = a.relu ? 0.f : -127.f, lo2 = a.relu2 ? 0.f : -127.f;
+  const float lo1h = a.relu ? 0.f : -__builtin_inff(), lo2h = a.relu2 ? 0.f : -__builtin_inff();
+
+  for (uint32_t tile = blockIdx.x * WAVES + wave; tile < tiles; tile += gridDim.x * WAVES) {
+    uint32_t m = __builtin_amdgcn_readfirstlane(a.tmask[tile]);
+    const uint32_t pos = tile * 32u + ln;
+    const uint32_t row = a.perm ? a.perm[pos] : pos;
+    const int32_t* __restrict__ nb = a.nbr + pos;
+    Acc acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[t][j] = 0;
+    while (m) {
+      int32_t idx[UNR];
+      int kk[UNR];     // this lane's offset of step u (16-byte rows: K-half 1 takes the pair's second offset)
+      int cnt = 0;
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        idx[u] = -1;
+        kk[u] = 0;
+        if (m) {   // wave-uniform
+          const int ka = __builtin_ctz(m);
+          m &= m - 1;
+          int k = ka;
+          bool have = true;
+          if (CHUNKS == 1) {
+            const int kb = m ? __builtin_ctz(m) : -1;
+            if (m) m &= m - 1;
+            have = lh == 0 || kb >= 0;
+            k = (lh && kb >= 0) ? kb : ka;
+          }
+          kk[u] = k;
+          if (have) idx[u] = nb[(size_t)k * a.nbr_ld];
+          cnt = u + 1;
+        }
+      }
+      v4i bf[UNR][KS];
+#pragma unroll
+      for (int u = 0; u < UNR; ++u)
+#pragma unroll
+        for (int ss = 0; ss < KS; ++ss) {
+          const int chunk = CHUNKS == 1 ? 0 : 2 * ss + lh;
+          const char* p = idx[u] >= 0 ? xb + (size_t)(uint32_t)idx[u] * ldb + chunk * 16 : zrow;
+          bf[u][ss] = u < cnt ? *reinterpret_cast<const v4i*>(p) : v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        if (u >= cnt) break;   // wave-uniform
+#pragma unroll
+        for (int ss = 0; ss < KS; ++ss) {
+          const int g = kk[u] * CHUNKS + (CHUNKS == 1 ? 0 : 2 * ss + lh);   // this lane's chunk of the weight sequence
+#pragma unroll
+          for (int t = 0; t < MT; ++t) {
+            const v4i af = wl[((g >> 1) * MT + t) * 64 + (g & 1) * 32 + ln];
+            acc[t] = Mma32<EL>::run(af, bf[u][ss], acc[t]);
+          }
+        }
+      }
+    }
+    // epilogue: lane (ln, lh) holds channels 32 t + 8 g + 4 lh .. + 3 of row `row`
+    if (row >= n) continue;
+    auto store_tile = [&](auto mode_c) {
+      constexpr int MODE = decltype(mode_c)::value;
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int co = t * 32 + g * 8 + lh * 4;
+          if (co >= cout_pad) continue;
+          const Acc4 piece = {acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
+          const float4 b4 = *reinterpret_cast<const float4*>(ep + co);
+          const float4 sc4 = *reinterpret_cast<const float4*>(ep + MT * 32 + co);
+          if constexpr (MODE == 1 || MODE == 3) {
+            uint32_t r4 = 0;
+            if constexpr (MODE == 3) r4 = *reinterpret_cast<const uint32_t*>(a.res + (size_t)row * a.res_ld + co);
+            *reinterpret_cast<uint32_t*>(a.out + (size_t)row * a.out_ld + co) =
+                epilogue_pack8<EL, MODE>(a, piece, b4, sc4, lo1, lo2, r4);
+          } else if constexpr (MODE == 2 || MODE == 4) {
+            v4h r4 = {0, 0, 0, 0};
+            if constexpr (MODE == 4)
+              r4 = *reinterpret_cast<const v4h*>(reinterpret_cast<const _Float16*>(a.res) + (size_t)row * a.res_ld + co);
+            *reinterpret_cast<v4h*>(reinterpret_cast<_Float16*>(a.out) + (size_t)row * a.out_ld + co) =
+                epilogue_pack16<EL, MODE>(piece, b4, sc4, lo1h, lo2h, r4);
+          } else {
+            epilogue_store<EL>(a, row, co, piece, b4, sc4);
+          }
+        }
+    };
+    switch (mode) {
+      case 1: store_tile(std::integral_constant<int, 1>{}); break;
+      case 2: store_tile(std::integral_constant<int, 2>{}); break;
+      case 3: store_tile(std::integral_constant<int, 3>{}); break;
+      case 4: store_tile(std::integral_constant<int, 4>{}); break;
+      default: store_tile(std::integral_constant<int, 0>{}); break;
+    }
+  }
+}
+
+template <int EL, int CHUNKS, int MT>
+static void launch_conv_tile(const ConvArgs& a, uint32_t n_hint, hipStream_t stream) {
+  // two workgroups of 8 waves per CU at most; fewer when the expected rows are fewer than that many tiles
+  const uint32_t tiles = ceil_div(n_hint ? n_hint : a.n_bound, 32u);
+  uint32_t blocks = ceil_div(tiles, 8u);
+  blocks = blocks < 1 ? 1 : blocks > 512 ? 512 : blocks;
+  const size_t lds = (size_t)a.steps32 * MT * 1024 + (size_t)MT * 32 * 8;
+  hipLaunchKernelGGL((k_conv_tile<EL, CHUNKS, MT>), dim3(blocks), dim3(512), lds, stream, a);
+}
+
+template <int EL>
+static bool dispatch_tile(int chunks, int mt, uint32_t n_hint, const ConvArgs& a, hipStream_t stream) {
+  if (mt == 1) {
+    switch (chunks) {
+      case 1: launch_conv_tile<EL, 1, 1>(a, n_hint, stream); return true;
+      case 2: launch_conv_tile<EL, 2, 1>(a, n_hint, stream); return true;
+      case 4: launch_conv_tile<EL, 4, 1>(a, n_hint, stream); return true;
+    }
+  } else if (mt == 2) {
+    switch (chunks) {
+      case 1: launch_conv_tile<EL, 1, 2>(a, n_hint, stream); return true;
+      case 2: launch_conv_tile<EL, 2, 2>(a, n_hint, stream); return true;
+    }
+  }
+  return false;
+}
+
 // SCN_CONV_IMPL=rows forces the plain row-split kernel (A/B measurements; it is also the fallback for
 // more than 128 output channels).
 static int conv_impl() {

@@ -19,6 +19,7 @@
 #include <string>
 #include <vector>
 
+#include "scn_conv_args.hpp"
 #include "scn_kernels.hpp"
 
 namespace scn {
@@ -164,6 +165,8 @@ struct RbSlot {
   uint32_t max_out = 0;
   int inverse_of = -1;   // >= 0: the strided rulebook this one swaps (SparseInverseConvolution)
   bool initialised = false;
+  bool want_plan = false;   // some convolution on this rulebook runs the tile-plan kernel
+  bool plan_sorted = false; // ... with the rows sorted by their offset sets (SCN_BUILD_SORTMASK)
 };
 
 }  // namespace scn
@@ -464,6 +467,10 @@ static bool build_engine(scn_engine& e) {
                      n.bias.empty() ? nullptr : n.bias.data(), comp))
           return false;
         const int ci = (int)e.convs.size();
+        if (slot.inverse_of < 0 && conv_tile_covers(*w)) {
+          slot.want_plan = true;
+          slot.plan_sorted = (e.flags & SCN_BUILD_SORTMASK) != 0;
+        }
         // input form the kernel needs
         Step st;
         st.kind = StepKind::Conv;
@@ -812,6 +819,10 @@ static int allocate_runtime(scn_engine& e) {
     // everything a build would allocate lazily is allocated here: forward() must not allocate
     int rc = s.subm ? s.rb.reserve_subm(false) : s.rb.reserve_sparse(e.coords[s.coord_out].grid, false);
     if (rc) return rc;
+    if (s.want_plan) {
+      rc = s.rb.reserve_plan(s.plan_sorted);
+      if (rc) return rc;
+    }
   }
   const bool keep_all = (e.flags & SCN_BUILD_KEEP_ALL) != 0;
   for (size_t t = 0; t < e.tensors.size(); ++t) {
@@ -928,8 +939,10 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
     case StepKind::RulebookSubm: {
       RbSlot& s = *e.rulebooks[st.rulebook];
       CoordSet& cs = e.coords[s.coord_in];
-      return s.rb.build_subm(cs.idx, cs.n_bound, cs.n_dev, cs.grid, s.ks, s.dil, cs.has_lookup ? &cs.lookup : nullptr,
-                             stream);
+      int rc = s.rb.build_subm(cs.idx, cs.n_bound, cs.n_dev, cs.grid, s.ks, s.dil, cs.has_lookup ? &cs.lookup : nullptr,
+                               stream);
+      if (rc == SCN_OK && s.want_plan) rc = s.rb.build_plan(s.plan_sorted, stream);
+      return rc;
     }
     case StepKind::RulebookSparse: {
       RbSlot& s = *e.rulebooks[st.rulebook];
@@ -938,6 +951,10 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
       int rc = s.rb.build_sparse(ci.idx, ci.n_bound, ci.n_dev, ci.grid, s.ks, s.stride, s.pad, s.dil,
                                  ci.has_lookup ? &ci.lookup : nullptr, stream);
       if (rc) return rc;
+      if (s.want_plan) {
+        rc = s.rb.build_plan(s.plan_sorted, stream);
+        if (rc) return rc;
+      }
       co.idx = s.rb.out_indices;
       co.n_dev = s.rb.n_out_dev();
       co.n_bound = s.rb.n_bound_out;
@@ -984,9 +1001,18 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
         io.b_requant_range = st.b_rq;
         io.relu_after_add = st.relu2;
       }
+      PlanView pv;
+      const TilePlan& tp = s.rb.plan;
+      const bool planned = s.want_plan && tp.built;
+      if (planned) {
+        pv.tmask = tp.tmask.as<uint32_t>();
+        if (tp.sorted) {
+          pv.perm = tp.perm.as<uint32_t>();
+          pv.nbr = tp.nbr.as<int32_t>();
+        }
+      }
       return conv_forward(*e.convs[st.conv], s.rb.nbr.as<int32_t>(), s.rb.ld, s.rb.n_out_dev(), s.rb.n_bound_out,
-                          s.rb.n_out_hint(), io,
-                          stream);
+                          s.rb.n_out_hint(), io, stream, planned ? &pv : nullptr);
     }
     case StepKind::Add: {
       const RtTensor& a = e.tensors[st.t_in];

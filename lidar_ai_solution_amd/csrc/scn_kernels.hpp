@@ -44,6 +44,21 @@ struct ConvGeom {
   int kvol;
 };
 
+// Tile plan of a rulebook: what lets a convolution skip the kernel offsets at which none of a 32-row tile's rows
+// has a neighbour (`sortmask` of the reference's loader, libraries/3DSparseConvolution/src/onnx-parser.hpp:35-37:
+// "skip more insignificance computations").  tmask[t] = OR of the rows' offset sets (bit k: nbr[k][row] >= 0).
+// A sorted plan also orders the rows by their offset set (stable radix sort of the sets as numbers), so that the
+// rows of a tile share most offsets: perm[j] = row at position j, nbr = the table in that order.  Results do not
+// depend on the plan: every row still adds its own products in offset order.
+struct TilePlan {
+  DevBuf keys, keys_sorted, rows, perm, tmask, nbr, temp;
+  size_t temp_bytes = 0;
+  uint32_t cap_rows = 0;   // positions allocated (multiple of 32)
+  bool reserved_sorted = false;
+  bool sorted = false;     // what the last build produced
+  bool built = false;
+};
+
 // Rulebook object (= scn_rulebook of the C ABI).
 struct Rulebook {
   uint32_t max_in = 0, max_out = 0;
@@ -66,6 +81,7 @@ struct Rulebook {
   uint32_t n_bound_in = 0, n_bound_out = 0;
   bool built = false;
   bool bitmap_precleared = false;  // the next build_sparse finds its output bitmap already zeroed
+  TilePlan plan;
 
   bool init(uint32_t max_in_, uint32_t max_out_, int kvol);
   int reserve_sparse(const int out_grid[3], bool need_own_in_table);
@@ -78,6 +94,9 @@ struct Rulebook {
   // the rulebook of SparseInverseConvolution: fwd (strided, built) with inputs and outputs swapped; n_in_dev
   // (nullable) is the device-side row count of fwd's input, which becomes this rulebook's output count
   int build_inverse(const Rulebook& fwd, const uint32_t* n_in_dev, hipStream_t stream);
+  // tile plan of the table built last (kernel volumes up to 31); reserve_plan allocates, build_plan only launches
+  int reserve_plan(bool sorted);
+  int build_plan(bool sorted, hipStream_t stream);
   CoordLookup out_lookup() const;  // strided: rows of the output tensor from bitmap ranks
   int pairs(int32_t* pair_in, int32_t* pair_out, int64_t* offsets, uint64_t capacity, hipStream_t stream);
   const uint32_t* n_out_dev() const { return counters.as<uint32_t>(); }
@@ -102,8 +121,10 @@ struct ConvWeights {
 };
 
 // n_hint: expected row count (0 = unknown), only used to choose the launch configuration
+struct PlanView;
 int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, const uint32_t* n_out_dev,
-                 uint32_t n_bound, uint32_t n_hint, const scn_conv_io& io, hipStream_t stream);
+                 uint32_t n_bound, uint32_t n_hint, const scn_conv_io& io, hipStream_t stream,
+                 const PlanView* plan = nullptr);
 
 int set_count(uint32_t* dst, const uint32_t* n_dev, uint32_t n_bound, hipStream_t stream);
 int fill_u32(void* p, uint32_t value, size_t count, hipStream_t stream);

@@ -127,7 +127,7 @@ class Engine:
 
     @classmethod
     def from_graph(cls, graph: Graph, precision="fp16", keep_all: bool = False,
-                   with_auxiliary_stream: bool = False) -> "Engine":
+                   with_auxiliary_stream: bool = False, sortmask: bool = False) -> "Engine":
         """Drives the EngineBuilder calls (push_input / push_sparse_conv / ... / build) node by node,
         the way `onnx-parser.cpp:116-230` does."""
         L = capi.lib()
@@ -176,7 +176,8 @@ class Engine:
                 tmap[n.outputs[0]] = out
             for name in graph.outputs:
                 capi.check(L.scn_builder_push_output(b, tmap[name]))
-            flags = (capi.BUILD_KEEP_ALL if keep_all else 0) | (capi.BUILD_AUX_STREAM if with_auxiliary_stream else 0)
+            flags = (capi.BUILD_KEEP_ALL if keep_all else 0) | (capi.BUILD_AUX_STREAM if with_auxiliary_stream else 0) | \
+                    (capi.BUILD_SORTMASK if sortmask else 0)
             h = L.scn_builder_build(b, _prec(precision), flags, None)
         finally:
             L.scn_builder_destroy(b)
