@@ -881,16 +881,25 @@ __global__ __launch_bounds__(64 * WAVES, AHEAD > 1 ? 2 : conv_lds_min_waves(CHUN
 //   * positions of a sorted plan are not rows: the epilogue stores (and reads the residual of) row perm[pos].
 // Results are bit-identical to the other kernels: a row's products are added in offset order, integers exactly,
 // fp16 products in fp32 with zero terms left out.
+// waves per SIMD the tile-plan kernel is compiled for: eight (64 registers, four workgroups per CU) where the
+// weights leave room for four workgroups' copies in LDS, four otherwise
+constexpr int conv_tile_min_waves(int chunks, int mt) { return (mt == 1 && chunks <= 2) ? 8 : 4; }
+
 template <int EL, int CHUNKS, int MT>
-__global__ __launch_bounds__(512, 4) void k_conv_tile(const ConvArgs a) {
+__global__ __launch_bounds__(512, conv_tile_min_waves(CHUNKS, MT)) void k_conv_tile(const ConvArgs a) {
   using Acc = typename Mma32<EL>::Acc;
   using Acc4 = typename Mma32<EL>::Acc4;
   constexpr int WAVES = 8;
   constexpr int KS = CHUNKS >= 2 ? CHUNKS / 2 : 1;   // MFMAs per offset and output tile (16-byte rows: half of one)
-  constexpr int UNR = CHUNKS >= 4 ? 2 : 4;           // offsets (16-byte rows: offset pairs) in flight per step
+  constexpr int UNR = (CHUNKS >= 4 || conv_tile_min_waves(CHUNKS, MT) >= 8) ? 2 : 4;   // offsets (16-byte rows: offset pairs) in flight per step
   extern __shared__ v4i wl[];                        // [steps32][MT][64] A fragments, then bias[MT*32], scale[MT*32]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, ln = lane & 31, lh = lane >> 5;
   const int nfrag = a.steps32 * MT * 64;
+  const uint32_t n = eff_n(a.n_out_dev, a.n_bound);
+  const uint32_t tiles = (n + 31u) >> 5;
+  // the first tile's mask is on its way while the weights are copied
+  uint32_t tile = blockIdx.x * WAVES + wave;
+  uint32_t m_next = tile < tiles ? a.tmask[tile] : 0u;
   {
     const v4i* __restrict__ src = reinterpret_cast<const v4i*>(a.wfrag32);
     for (int i = tid; i < nfrag; i += 64 * WAVES) wl[i] = src[i];
@@ -904,8 +913,6 @@ __global__ __launch_bounds__(512, 4) void k_conv_tile(const ConvArgs a) {
   }
   __syncthreads();
 
-  const uint32_t n = eff_n(a.n_out_dev, a.n_bound);
-  const uint32_t tiles = (n + 31u) >> 5;
   const uint32_t ldb = a.x_ld_bytes;
   const char* __restrict__ xb = a.x;
   const char* __restrict__ zrow = a.zrow;
@@ -920,8 +927,12 @@ __global__ __launch_bounds__(512, 4) void k_conv_tile(const ConvArgs a) {
   const float lo1 = a.relu ? 0.f : -127.f, lo2 = a.relu2 ? 0.f : -127.f;
   const float lo1h = a.relu ? 0.f : -__builtin_inff(), lo2h = a.relu2 ? 0.f : -__builtin_inff();
 
-  for (uint32_t tile = blockIdx.x * WAVES + wave; tile < tiles; tile += gridDim.x * WAVES) {
-    uint32_t m = __builtin_amdgcn_readfirstlane(a.tmask[tile]);
+  for (; tile < tiles; tile += gridDim.x * WAVES) {
+    uint32_t m = __builtin_amdgcn_readfirstlane(m_next);
+    {
+      const uint32_t nt = tile + gridDim.x * WAVES;   // the next tile's mask arrives during this tile
+      m_next = nt < tiles ? a.tmask[nt] : 0u;
+    }
     const uint32_t pos = tile * 32u + ln;
     const uint32_t row = a.perm ? a.perm[pos] : pos;
     const int32_t* __restrict__ nb = a.nbr + pos;
@@ -1018,10 +1029,12 @@ __global__ __launch_bounds__(512, 4) void k_conv_tile(const ConvArgs a) {
 
 template <int EL, int CHUNKS, int MT>
 static void launch_conv_tile(const ConvArgs& a, uint32_t n_hint, hipStream_t stream) {
-  // two workgroups of 8 waves per CU at most; fewer when the expected rows are fewer than that many tiles
+  // as many workgroups of 8 waves as fit the GPU at once (two or four per CU); fewer when the expected rows
+  // are fewer than that many tiles
   const uint32_t tiles = ceil_div(n_hint ? n_hint : a.n_bound, 32u);
+  const uint32_t resident = 256u * (conv_tile_min_waves(CHUNKS, MT) / 2);
   uint32_t blocks = ceil_div(tiles, 8u);
-  blocks = blocks < 1 ? 1 : blocks > 512 ? 512 : blocks;
+  blocks = blocks < 1 ? 1 : blocks > resident ? resident : blocks;
   const size_t lds = (size_t)a.steps32 * MT * 1024 + (size_t)MT * 32 * 8;
   hipLaunchKernelGGL((k_conv_tile<EL, CHUNKS, MT>), dim3(blocks), dim3(512), lds, stream, a);
 }

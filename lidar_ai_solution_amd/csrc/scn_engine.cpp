@@ -467,9 +467,12 @@ static bool build_engine(scn_engine& e) {
                      n.bias.empty() ? nullptr : n.bias.data(), comp))
           return false;
         const int ci = (int)e.convs.size();
-        if (slot.inverse_of < 0 && conv_tile_covers(*w)) {
+        // sortmask: the narrow layers run on sorted tile plans.  (Without the switch no plan is built: in row
+        // order the tile-plan kernel is level with the LDS-staged one, and the masks would cost the first
+        // rulebook of a frame 9 us on the critical path.)
+        if ((e.flags & SCN_BUILD_SORTMASK) && slot.inverse_of < 0 && conv_tile_covers(*w)) {
           slot.want_plan = true;
-          slot.plan_sorted = (e.flags & SCN_BUILD_SORTMASK) != 0;
+          slot.plan_sorted = true;
         }
         // input form the kernel needs
         Step st;
