@@ -99,6 +99,8 @@ _SIGNATURES = {
     "scn_add_relu": (C.c_int, [vp, C.c_int, C.c_float, C.c_float, vp, C.c_int, C.c_float, C.c_float, vp, C.c_int,
                                C.c_float, C.c_int, u32, u32, vp, vp]),
     "scn_scatter_dense": (C.c_int, [vp, C.c_int, C.c_float, u32, u32, vp, u32, vp, i5, vp, vp, vp]),
+    "scn_scatter_dense_layout": (C.c_int, [vp, C.c_int, C.c_float, u32, u32, vp, u32, vp, i5, vp, C.c_int, C.c_int,
+                                           C.c_int, C.c_float, vp, vp]),
     "scn_scatter_dense_map_cells": (C.c_size_t, [i5, vp]),
     "scn_scatter_dense_with_map": (C.c_int, [vp, C.c_int, C.c_float, u32, u32, vp, u32, vp, i5, vp, vp, vp, vp]),
     "scn_scatter_dense_noalloc_max_cells": (C.c_size_t, []),

@@ -322,6 +322,93 @@ int scatter_dense(const void* feat, int dtype, float range, uint32_t c, uint32_t
   return SCN_OK;
 }
 
+// The remaining dense forms of push_dense (libraries/3DSparseConvolution/libspconv/include/spconv/engine.hpp:26,
+// 114-123): int8 output and the vectorised layouts.  The sparse tensor [N, C] on the grid (D0, D1, D2), one of whose
+// axes is z (the first for "zyx" tensors, the last for "xyz" ones; the other two are H and W in their order), is the
+// 4-D tensor [1, C * Z, H, W] with channel c * Z + z (what the exporters' dense().view() / permute().reshape() tails
+// build).  NCHW32 stores it as [1, ceil(C Z / 32), H, W, 32] (groups of 32 channels innermost, zero padded),
+// NHWzC as [1, H, W, Z, C].  The closed engine's own definition of the two layouts is not in the reference's
+// sources; these follow the layout names.  One thread per (row, channel); the tensor is cleared first.
+struct DenseForm {
+  int layout;      // 1 strides (NCHW and its transposes), 2 NCHW32, 3 NHWzC
+  int zaxis;       // 0 or 2: which spatial axis is z
+  int C, Z, H, W;
+  DenseStrides st; // layout 1
+};
+
+__global__ __launch_bounds__(256) void k_scatter_form(const void* feat, int dtype, float scale, uint32_t ld,
+                                                      const int4* __restrict__ coords, uint32_t n_bound,
+                                                      const uint32_t* n_dev, DenseForm f, void* out, int out_dtype,
+                                                      float out_r) {
+  const uint32_t n = eff_n(n_dev, n_bound);
+  const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const uint32_t row = (uint32_t)(t / (uint32_t)f.C), c = (uint32_t)(t % (uint32_t)f.C);
+  if (row >= n) return;
+  const int4 p = coords[row];
+  if (p.x != 0 || p.y < 0 || p.y >= f.st.d0 || p.z < 0 || p.z >= f.st.d1 || p.w < 0 || p.w >= f.st.d2) return;
+  const float v = load_value(feat, dtype, (size_t)row * ld + c, scale, 0.f, 0.f);
+  size_t off;
+  if (f.layout == 1) {
+    off = (size_t)(c * f.st.sc + p.y * f.st.s0 + p.z * f.st.s1 + p.w * f.st.s2);
+  } else {
+    const int z = f.zaxis == 0 ? p.y : p.w;
+    const int h = f.zaxis == 0 ? p.z : p.y;
+    const int w = f.zaxis == 0 ? p.w : p.z;
+    if (f.layout == 2) {
+      const uint32_t cz = c * (uint32_t)f.Z + (uint32_t)z;
+      off = ((((size_t)(cz >> 5) * f.H + h) * f.W + w) << 5) + (cz & 31u);
+    } else {
+      off = (((size_t)h * f.W + w) * f.Z + z) * f.C + c;
+    }
+  }
+  store_value(out, out_dtype, off, v, out_r);
+}
+
+size_t scatter_dense_form_elements(const int dense_shape[5], int zaxis, int layout) {
+  const size_t C = dense_shape[1];
+  const size_t Z = dense_shape[2 + zaxis], H = dense_shape[zaxis == 0 ? 3 : 2], W = dense_shape[zaxis == 0 ? 4 : 3];
+  if (layout == 2) return (C * Z + 31) / 32 * 32 * H * W;
+  return C * Z * H * W;
+}
+
+int scatter_dense_form(const void* feat, int dtype, float range, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
+                       const uint32_t* n_dev, const int dense_shape[5], const int perm[5], int zaxis, int layout,
+                       int out_dtype, float out_range, void* out, hipStream_t stream) {
+  SCN_REQUIRE(out && dense_shape, SCN_ERR_INVALID, "scatter_dense: null pointer");
+  SCN_REQUIRE(dense_shape[0] == 1 && (uint32_t)dense_shape[1] == c && c > 0, SCN_ERR_INVALID,
+              "scatter_dense: output_shape must be [1, C=%u, D0, D1, D2]", c);
+  SCN_REQUIRE(layout >= 1 && layout <= 3 && (zaxis == 0 || zaxis == 2), SCN_ERR_INVALID, "scatter_dense: bad layout");
+  SCN_REQUIRE(out_dtype == SCN_DTYPE_FP16 || (out_dtype == SCN_DTYPE_INT8 && out_range > 0.f), SCN_ERR_INVALID,
+              "scatter_dense: the output is fp16, or int8 with a dynamic range");
+  DenseForm f{};
+  f.layout = layout;
+  f.zaxis = zaxis;
+  f.C = (int)c;
+  f.Z = dense_shape[2 + zaxis];
+  f.H = dense_shape[zaxis == 0 ? 3 : 2];
+  f.W = dense_shape[zaxis == 0 ? 4 : 3];
+  int64_t dstride[5] = {0, 0, 0, 0, 0};
+  size_t numel = 0;
+  if (layout == 1) {
+    SCN_REQUIRE(dense_layout(dense_shape, perm, dstride, &numel), SCN_ERR_INVALID, "scatter_dense: bad permutation");
+  } else {
+    SCN_REQUIRE(perm == nullptr, SCN_ERR_INVALID, "scatter_dense: a vectorised layout takes no Transpose");
+    numel = scatter_dense_form_elements(dense_shape, zaxis, layout);
+  }
+  f.st = DenseStrides{dstride[1], dstride[2], dstride[3], dstride[4], dense_shape[2], dense_shape[3], dense_shape[4]};
+  const size_t bytes = numel * (out_dtype == SCN_DTYPE_INT8 ? 1 : 2);
+  SCN_REQUIRE(bytes % 4 == 0, SCN_ERR_UNSUPPORTED, "scatter_dense: tensor size %zu is not a multiple of 4 bytes", bytes);
+  int rc = fill_u32(out, 0u, bytes / 4, stream);
+  if (rc || n == 0) return rc;
+  SCN_REQUIRE(feat && idx, SCN_ERR_INVALID, "scatter_dense: null input");
+  const size_t total = (size_t)n * c;
+  hipLaunchKernelGGL(k_scatter_form, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, feat, dtype,
+                     range > 0.f ? range / 127.f : 1.f, ld, (const int4*)idx, n, n_dev, f, out, out_dtype,
+                     out_range > 0.f ? 127.f / out_range : 1.f);
+  SCN_HIP(hipGetLastError());
+  return SCN_OK;
+}
+
 // Stand-alone dense permute of a 5-D fp16 tensor (used only when the Transpose is not fused into
 // the scatter): out[o0..o4] = in[index with dim perm[j] = o_j].
 struct Permute5 {
@@ -419,6 +506,14 @@ int scn_scatter_dense(const void* feat_dev, int dtype, float dynamic_range, uint
                       const int perm[5], void* out_fp16_dev, void* stream) {
   return scatter_dense(feat_dev, dtype, dynamic_range, c, ld, indices_dev, n, n_dev, dense_shape, perm, out_fp16_dev,
                        (hipStream_t)stream);
+}
+
+int scn_scatter_dense_layout(const void* feat_dev, int dtype, float dynamic_range, uint32_t c, uint32_t ld,
+                             const int32_t* indices_dev, uint32_t n, const uint32_t* n_dev, const int dense_shape[5],
+                             const int perm[5], int z_axis, int output_layout, int out_dtype, float out_dynamic_range,
+                             void* out_dev, void* stream) {
+  return scatter_dense_form(feat_dev, dtype, dynamic_range, c, ld, indices_dev, n, n_dev, dense_shape, perm, z_axis,
+                            output_layout, out_dtype, out_dynamic_range, out_dev, (hipStream_t)stream);
 }
 
 size_t scn_scatter_dense_map_cells(const int dense_shape[5], const int perm[5]) {

@@ -63,6 +63,7 @@ struct NodeDesc {
   int in_spatial[3] = {0, 0, 0};
   std::vector<int> out_shape;
   float dense_range = 0.f;
+  int layout = 1;  // spconv::TensorLayout: 1 NCHW, 2 NCHW32, 3 NHWzC
   // reshape / transpose
   std::vector<int64_t> dims;
 };
@@ -118,6 +119,7 @@ struct RtTensor {
   void* data = nullptr;
   DevBuf acc;          // raw accumulators (keep-all mode)
   std::vector<int64_t> shape;  // dense
+  bool fixed_form = false;     // dense tensor in a vectorised layout: a following Reshape keeps this shape
   int view_of = -1;    // dense view of another tensor (reshape / fused transpose)
   bool materialised = false;  // false: fused away, never written
 };
@@ -152,6 +154,8 @@ struct Step {
   int dense_shape[5] = {1, 0, 0, 0, 0};
   int perm[5] = {0, 1, 2, 3, 4};
   bool has_perm = false;
+  bool form = false;           // int8 output or a vectorised layout: scatter_dense_form
+  int form_layout = 1, zaxis = 0;
   // profiling
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   float last_ms = 0.f;
@@ -675,10 +679,38 @@ static bool build_engine(scn_engine& e) {
         for (int j = 0; j < 5; ++j) st.dense_shape[j] = n.out_shape[j];
         int t_out = n.out;
         std::vector<int64_t> shape(n.out_shape.begin(), n.out_shape.end());
+        const bool out_i8 = n.dense_range > 0.f && e.precision == SCN_PRECISION_INT8;
+        st.form = out_i8 || n.layout != 1;
+        st.form_layout = n.layout;
+        st.zaxis = n.format == "xyz" ? 2 : 0;
+        int c1 = single_consumer(n.out);
+        const bool next_is_transpose = c1 >= 0 && nodes[c1].op == Op::Transpose && nodes[c1].dims.size() == 5;
+        if (n.layout != 1) {
+          // a vectorised layout is defined on the [1, C * Z, H, W] view; the exporter's tail for "xyz" tensors
+          // brings z to the front with Transpose (0, 1, 4, 2, 3) first, which the layout already accounts for
+          for (size_t u = i + 1; u < nodes.size(); ++u)
+            if (nodes[u].op == Op::Transpose && !nodes[u].in.empty() && nodes[u].in[0] == n.out) {
+              const auto& d = nodes[u].dims;
+              const bool z_front = st.zaxis == 2 && d.size() == 5 && d[0] == 0 && d[1] == 1 && d[2] == 4 && d[3] == 2 && d[4] == 3;
+              if (!z_front || (int)u != c1) {
+                set_error("node %s: a %s output cannot be transposed", n.name.c_str(), n.layout == 2 ? "NCHW32" : "NHWzC");
+                return false;
+              }
+            }
+          if (next_is_transpose) {
+            fused_away[c1] = true;
+            e.tensors[n.out].dense = true;
+            t_out = nodes[c1].out;
+            st.label += "+" + nodes[c1].name;
+          }
+          const int64_t C = n.out_shape[1], Z = n.out_shape[2 + st.zaxis], H = n.out_shape[st.zaxis == 0 ? 3 : 2],
+                        W = n.out_shape[st.zaxis == 0 ? 4 : 3];
+          if (n.layout == 2) shape = {1, (C * Z + 31) / 32, H, W, 32};
+          else shape = {1, H, W, Z, C};
+        }
         // fold a following Transpose (and Reshape views) into the scatter
-        if (!keep_all) {
-          int c1 = single_consumer(n.out);
-          if (c1 >= 0 && nodes[c1].op == Op::Transpose && nodes[c1].dims.size() == 5) {
+        if (!keep_all && n.layout == 1) {
+          if (next_is_transpose) {
             bool okp = true;
             bool seen[5] = {false, false, false, false, false};
             for (int j = 0; j < 5; ++j) {
@@ -702,7 +734,9 @@ static bool build_engine(scn_engine& e) {
         }
         RtTensor& o = e.tensors[t_out];
         o.dense = true;
-        o.dtype = SCN_DTYPE_FP16;
+        o.dtype = out_i8 ? SCN_DTYPE_INT8 : SCN_DTYPE_FP16;
+        o.range = out_i8 ? n.dense_range : 0.f;
+        o.fixed_form = n.layout != 1;
         o.shape = shape;
         o.materialised = true;
         st.t_out = t_out;
@@ -714,6 +748,18 @@ static bool build_engine(scn_engine& e) {
         if (!x.dense) {
           set_error("node %s: Reshape needs a dense input", n.name.c_str());
           return false;
+        }
+        if (x.fixed_form) {
+          // the tensor is already the vectorised form of the network's final 4-D tensor: an alias with that shape
+          RtTensor& o = e.tensors[n.out];
+          o.dense = true;
+          o.dtype = x.dtype;
+          o.range = x.range;
+          o.shape = x.shape;
+          o.fixed_form = true;
+          o.view_of = x.view_of >= 0 ? x.view_of : n.in[0];
+          o.materialised = true;
+          break;
         }
         int64_t numel = 1, known = 1;
         int infer = -1;
@@ -732,6 +778,7 @@ static bool build_engine(scn_engine& e) {
         RtTensor& o = e.tensors[n.out];
         o.dense = true;
         o.dtype = x.dtype;
+        o.range = x.range;
         o.shape = shape;
         o.view_of = x.view_of >= 0 ? x.view_of : n.in[0];
         o.materialised = true;
@@ -740,8 +787,8 @@ static bool build_engine(scn_engine& e) {
       case Op::Transpose: {
         // reached only when the Transpose was not folded into the preceding ScatterDense
         RtTensor& x = e.tensors[n.in[0]];
-        if (!x.dense || x.shape.size() != 5 || n.dims.size() != 5) {
-          set_error("node %s: Transpose needs a dense 5-D input and 5 dims", n.name.c_str());
+        if (!x.dense || x.shape.size() != 5 || n.dims.size() != 5 || x.fixed_form || x.dtype != SCN_DTYPE_FP16) {
+          set_error("node %s: Transpose needs a dense 5-D fp16 input in the NCHW layout and 5 dims", n.name.c_str());
           return false;
         }
         Step st;
@@ -835,7 +882,8 @@ static int allocate_runtime(scn_engine& e) {
       if (x.view_of >= 0) continue;
       size_t numel = 1;
       for (auto v : x.shape) numel *= (size_t)v;
-      if (x.buf.bytes < numel * 2 && !x.buf.alloc(numel * 2)) return SCN_ERR_HIP;
+      const size_t dbytes = (numel * (x.dtype == SCN_DTYPE_INT8 ? 1 : 2) + 15) & ~(size_t)15;
+      if (x.buf.bytes < dbytes && !x.buf.alloc(dbytes)) return SCN_ERR_HIP;
       x.data = x.buf.p;
       continue;
     }
@@ -852,7 +900,7 @@ static int allocate_runtime(scn_engine& e) {
   e.dense_maps.resize(e.steps.size());
   for (size_t si = 0; si < e.steps.size(); ++si) {
     const Step& st = e.steps[si];
-    if (st.kind != StepKind::Dense) continue;
+    if (st.kind != StepKind::Dense || st.form) continue;
     const size_t cells = scatter_dense_map_cells(st.dense_shape, st.has_perm ? st.perm : nullptr);
     if (cells && e.dense_maps[si].bytes < cells * 4 && !e.dense_maps[si].alloc(cells * 4)) return SCN_ERR_HIP;
   }
@@ -912,7 +960,7 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
         } else if (s2.kind == StepKind::RulebookSparse) {
           Rulebook& rb = e.rulebooks[s2.rulebook]->rb;
           if (rb.bitmap.p && rb.bitmap_words && add(rb.bitmap.p, rb.bitmap_words, 0u)) rb.bitmap_precleared = true;
-        } else if (s2.kind == StepKind::Dense) {
+        } else if (s2.kind == StepKind::Dense && !s2.form) {
           RtTensor& o = e.tensors[s2.t_out];
           size_t numel = 1;
           for (int j = 0; j < 5; ++j) numel *= (size_t)s2.dense_shape[j];
@@ -1037,6 +1085,9 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
       const RtTensor& x = e.tensors[st.t_in];
       RtTensor& o = e.tensors[st.t_out];
       const CoordSet& cs = e.coords[x.coord];
+      if (st.form)
+        return scatter_dense_form(x.data, x.dtype, x.range, (uint32_t)x.c, x.ld, cs.idx, cs.n_bound, cs.n_dev, st.dense_shape,
+                                  st.has_perm ? st.perm : nullptr, st.zaxis, st.form_layout, o.dtype, o.range, o.data, stream);
       const size_t si = (size_t)(&st - e.steps.data());
       const int pre = si < e.dense_precleared.size() ? e.dense_precleared[si] : 0;
       int32_t* map = si < e.dense_maps.size() ? e.dense_maps[si].as<int32_t>() : nullptr;
@@ -1366,8 +1417,12 @@ int scn_builder_push_dense(scn_builder* b, const char* name, int x, const char* 
     set_error("push_dense(%s): invalid arguments", name ? name : "");
     return -1;
   }
-  if (output_layout != 0 && output_layout != 1) {
-    set_error("push_dense(%s): only the NCHW output layout is supported (got %d)", name ? name : "", output_layout);
+  if (output_layout < 0 || output_layout > 3) {
+    set_error("push_dense(%s): unknown output layout %d", name ? name : "", output_layout);
+    return -1;
+  }
+  if (n_output_shape != 5) {
+    set_error("push_dense(%s): output_shape must be [1, C, D0, D1, D2]", name ? name : "");
     return -1;
   }
   NodeDesc n;
@@ -1377,8 +1432,8 @@ int scn_builder_push_dense(scn_builder* b, const char* name, int x, const char* 
   n.format = format ? format : "";
   copy3(n.in_spatial, input_spatial_shape, 0);
   n.out_shape.assign(output_shape, output_shape + n_output_shape);
-  n.dense_range = 0.f;  // int8 dense output is not supported: the dense tensor is always fp16
-  (void)input_dynamic_range;
+  n.dense_range = input_dynamic_range > 0.f ? input_dynamic_range : 0.f;  // > 0: int8 output under an int8 engine
+  n.layout = output_layout == 0 ? 1 : output_layout;
   n.out = b->new_tensor(output_name, (int)b->nodes.size());
   b->nodes.push_back(std::move(n));
   return b->nodes.back().out;

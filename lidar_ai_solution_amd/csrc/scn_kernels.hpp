@@ -164,6 +164,13 @@ int scatter_dense_build_map(const int32_t* idx, uint32_t n, const uint32_t* n_de
 // 16-byte stores); 0 when the layout does not qualify (channel axis not outermost, plane not a multiple of 8).
 size_t scatter_dense_map_cells(const int dense_shape[5], const int perm[5]);
 
+// the other forms of the dense output: layout 1 NCHW (with an optional Transpose), 2 NCHW32, 3 NHWzC of the
+// [1, C * Z, H, W] view (zaxis 0: "zyx" tensors, 2: "xyz"), fp16 or int8 (out_range = its dynamic range)
+size_t scatter_dense_form_elements(const int dense_shape[5], int zaxis, int layout);
+int scatter_dense_form(const void* feat, int dtype, float range, uint32_t c, uint32_t ld, const int32_t* idx, uint32_t n,
+                       const uint32_t* n_dev, const int dense_shape[5], const int perm[5], int zaxis, int layout,
+                       int out_dtype, float out_range, void* out, hipStream_t stream);
+
 int permute_dense(const void* in, const int64_t in_shape[5], const int perm[5], void* out, hipStream_t stream);
 
 }  // namespace scn

@@ -272,6 +272,24 @@ def scatter_dense(feat: np.ndarray, indices: np.ndarray, dims) -> np.ndarray:
     return dense
 
 
+def dense_to_layout(dense: np.ndarray, fmt: str, layout: str) -> np.ndarray:
+    """[1, C, D0, D1, D2] -> the vectorised layouts of push_dense (engine.hpp:26): first the 4-D tensor
+    [1, C * Z, H, W] the exporters' tails build (channel c * Z + z; z is the first spatial axis of "zyx" tensors,
+    the last of "xyz" ones), then NCHW32 = [1, ceil(CZ / 32), H, W, 32] zero padded, NHWzC = [1, H, W, Z, C]."""
+    if fmt == "xyz":
+        dense = np.transpose(dense, (0, 1, 4, 2, 3))      # [1, C, Z, H, W]
+    _, c, z, h, w = dense.shape
+    if layout == "NHWzC":
+        return np.ascontiguousarray(np.transpose(dense, (0, 3, 4, 2, 1)))
+    if layout != "NCHW32":
+        raise ValueError(layout)
+    flat = np.ascontiguousarray(dense).reshape(1, c * z, h, w)
+    groups = (c * z + 31) // 32
+    pad = np.zeros((1, groups * 32, h, w), dense.dtype)
+    pad[:, :c * z] = flat
+    return np.ascontiguousarray(pad.reshape(1, groups, 32, h, w).transpose(0, 1, 3, 4, 2))
+
+
 # ------------------------------------------------------------------------------- graph walk
 class SparseT:
     """features (fp16, or int8 with its dynamic range `rng`), indices, grid."""
@@ -451,12 +469,30 @@ def run_graph(graph, features_f16: np.ndarray, indices: np.ndarray, grid, precis
                 rec.update(out=out, range=X.rng)
         elif n.op_type == "ScatterDense":
             X = T[n.inputs[0]]
-            feat = X.feat if X.feat.dtype == np.float16 else dequantize(X.feat, float(X.rng))
             oshape = [int(v) for v in n.attrs["output_shape"]]
-            dense = scatter_dense(feat, X.indices, oshape[2:5])
+            out_rng = float(n.attrs.get("input_dynamic_range", 0.0) or 0.0)
+            layout = n.attrs.get("output_layout", "") or "NCHW"
+            if out_rng > 0 and precision == "int8":
+                # int8 dense output (push_dense's input_dynamic_range, engine.hpp:121): the fp32 value of every
+                # element, quantised with the node's range
+                val = X.feat.astype(np.float32) if X.feat.dtype == np.float16 else \
+                    X.feat.astype(np.float32) * (f32(X.rng) / f32(127.0))
+                dense = scatter_dense(quantize_f32(val, out_rng), X.indices, oshape[2:5])
+            else:
+                feat = X.feat if X.feat.dtype == np.float16 else dequantize(X.feat, float(X.rng))
+                dense = scatter_dense(feat, X.indices, oshape[2:5])
+            if layout != "NCHW":
+                dense = dense_to_layout(dense, n.attrs.get("format", "zyx"), layout)
+                T["__fixed_form__" + n.outputs[0]] = True
             T[n.outputs[0]] = dense
             if rec is not None:
                 rec.update(out=dense)
+        elif n.op_type in ("Reshape", "Transpose") and T.get("__fixed_form__" + n.inputs[0]):
+            # a tensor in a vectorised layout already is the final tensor: the exporter's tail leaves it as it is
+            T[n.outputs[0]] = T[n.inputs[0]]
+            T["__fixed_form__" + n.outputs[0]] = True
+            if rec is not None:
+                rec.update(out=T[n.outputs[0]])
         elif n.op_type == "Reshape":
             T[n.outputs[0]] = np.ascontiguousarray(T[n.inputs[0]]).reshape([int(v) for v in n.attrs["dims"]])
             if rec is not None:

@@ -540,6 +540,40 @@ def test_cpp_lidar_scn_glue_one_graph_for_voxelization_and_backbone(aux, nuscene
     assert np.array_equal(got.view(np.uint16), want.view(np.uint16)) and np.count_nonzero(got) > 100000
 
 
+@pytest.mark.parametrize("kind,layout,int8_out", [("centerpoint", "NCHW32", True), ("centerpoint", "NCHW", True),
+                                                  ("bevfusion", "NHWzC", False), ("bevfusion", "NCHW32", True)])
+def test_dense_output_layout_and_int8_through_the_engine(kind, layout, int8_out, centerpoint_input, bevfusion_input, tmp_path):
+    """ScatterDense's output_layout / input_dynamic_range attributes (src/onnx-parser.cpp:196-203) from a model file:
+    the engine's dense output equals the oracle walk's bit for bit (int8 plans, the last convolution stored int8 at
+    the dense node's range when the output is int8)."""
+    feats, idx = centerpoint_input if kind == "centerpoint" else bevfusion_input
+    grid = GRID_ZYX if kind == "centerpoint" else GRID_XYZ
+    make = graphs.centerpoint_scn if kind == "centerpoint" else graphs.bevfusion_scn
+    g16, _ = make(seed=3)
+    amax = _oracle_calibration(g16, feats, idx, grid)
+    g8, tags8 = make(seed=3)
+    graphs.apply_int8_plan(g8, tags8, amax, "all-int8")
+    dense = [n for n in g8.nodes if n.op_type == "ScatterDense"][0]
+    dense.attrs["output_layout"] = layout
+    if int8_out:
+        dense.attrs["input_dynamic_range"] = float(amax[dense.inputs[0]])
+    note(f"{kind}-shaped int8 graph with a {layout} {'int8' if int8_out else 'fp16'} dense output")
+    path = str(tmp_path / "layout.scn.onnx")
+    onnx_dialect.save(g8, path)
+    eng = Engine.from_onnx(path, "int8")
+    _run_engine(eng, feats, idx, grid)
+    out = eng.output(0)
+    want = O.run_graph(g8, feats, idx, grid, "int8")[g8.outputs[0]]
+    got = out.torch().cpu().numpy()
+    assert out.dtype == (capi.DTYPE_INT8 if int8_out else capi.DTYPE_FP16)
+    expect_shape = {"NCHW32": (1, 8, 180, 180, 32), "NHWzC": (1, 180, 180, 2, 128), "NCHW": (1, 256, 180, 180)}[layout]
+    assert tuple(got.shape) == expect_shape == tuple(want.shape), (got.shape, want.shape)
+    assert got.dtype == want.dtype and np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    assert np.count_nonzero(got) > 100000
+    if int8_out:
+        assert np.float32(out.dynamic_range) == np.float32(dense.attrs["input_dynamic_range"])
+
+
 def test_legacy_single_call_interface_and_precision_overrides(cp_models, centerpoint_input, tmp_path):
     """The older engine interface (forward(shapes, types, pointers, ...) -> DTensor*, set_node_precision_by*,
     reconfigure) through the C++ caller built against include/legacy/spconv/engine.hpp, and the loader's

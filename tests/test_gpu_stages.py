@@ -517,6 +517,52 @@ def test_scatter_dense_with_row_map():
                 assert np.array_equal(out.cpu().numpy().view(np.uint16), ref.view(np.uint16))
 
 
+@pytest.mark.parametrize("fmt", ["zyx", "xyz"])
+def test_dense_output_layouts_and_int8(fmt):
+    """push_dense's other output forms (engine.hpp:26,114-123): int8 output in the NCHW layout (with and without a
+    Transpose), and NCHW32 / NHWzC of the [1, C * Z, H, W] view, fp16 and int8, against numpy reshapes of the
+    oracle's NCHW tensor."""
+    L = capi.lib()
+    rng = np.random.default_rng(17)
+    dims = (2, 36, 40) if fmt == "zyx" else (36, 40, 2)
+    zaxis = 0 if fmt == "zyx" else 2
+    n = 1500
+    vol = int(np.prod(dims))
+    lin = np.sort(rng.choice(vol, n, replace=False))
+    idx = np.zeros((n, 4), np.int32)
+    idx[:, 1], idx[:, 2], idx[:, 3] = lin // (dims[1] * dims[2]), (lin // dims[2]) % dims[1], lin % dims[2]
+    d_idx = to_dev(idx)
+    for c in (24, 128):      # 24 * 2 = 48 channels: NCHW32 pads the second group
+        ld = (c + 15) // 16 * 16
+        for in_dtype in (capi.DTYPE_INT8, capi.DTYPE_FP16):
+            if in_dtype == capi.DTYPE_INT8:
+                feat = np.zeros((n, ld), np.int8); feat[:, :c] = rng.integers(-127, 128, (n, c)); in_rng = 3.3
+                val = feat[:, :c].astype(np.float32) * (np.float32(in_rng) / np.float32(127))
+            else:
+                feat = np.zeros((n, ld), np.float16); feat[:, :c] = rng.standard_normal((n, c)); in_rng = 0.0
+                val = feat[:, :c].astype(np.float32)
+            d_feat = to_dev(feat)
+            for out_i8 in (False, True):
+                out_rng = 2.9 if out_i8 else 0.0
+                rows = O.quantize_f32(val, out_rng) if out_i8 else val.astype(np.float16)
+                nchw = O.scatter_dense(rows, idx, dims)
+                for layout, name in ((1, "NCHW"), (2, "NCHW32"), (3, "NHWzC")):
+                    perms = [None, (0, 1, 4, 2, 3)] if layout == 1 else [None]
+                    for perm in perms:
+                        want = nchw if layout == 1 else O.dense_to_layout(nchw, fmt, name)
+                        if perm:
+                            want = np.ascontiguousarray(want.transpose(perm))
+                        note(f"dense {name} perm={perm} fmt={fmt} C={c} in={in_dtype} int8 out={out_i8}: {want.shape}")
+                        out = torch.full(want.shape, 3, dtype=torch.int8 if out_i8 else torch.float16, device=DEV)
+                        capi.check(L.scn_scatter_dense_layout(ptr(d_feat), in_dtype, in_rng, c, ld, ptr(d_idx), n, None,
+                                                              capi.i5(1, c, *dims), capi.i5(*perm) if perm else None, zaxis, layout,
+                                                              capi.DTYPE_INT8 if out_i8 else capi.DTYPE_FP16, out_rng, ptr(out), stream()))
+                        torch.cuda.synchronize()
+                        got = out.cpu().numpy()
+                        assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+                        assert np.count_nonzero(got) > n
+
+
 def test_memset_kernel_any_alignment_and_inside_a_graph():
     """scn_memset_async (Tensor::memset of the C++ header): byte ranges with unaligned heads and tails, and
     recorded into a HIP graph that is replayed with other work in between."""
