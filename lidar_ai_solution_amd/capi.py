@@ -60,6 +60,7 @@ LOG_CALLBACK = C.CFUNCTYPE(None, C.c_char_p, C.c_int, C.c_char_p, C.c_int, vp)
 _SIGNATURES = {
     "scn_version": (C.c_int, []),
     "scn_last_error": (C.c_char_p, []),
+    "scn_device_bytes_in_use": (C.c_size_t, []),
     "scn_set_log_level": (None, [C.c_int]),
     "scn_get_log_level": (C.c_int, []),
     "scn_set_log_callback": (None, [LOG_CALLBACK, vp]),

@@ -41,6 +41,11 @@ void log_message(const char* file, int line, int level, const char* fmt, ...) {
   emit(file, line, level, buf);
 }
 
+std::atomic<size_t>& device_bytes_counter() {
+  static std::atomic<size_t> bytes{0};
+  return bytes;
+}
+
 void set_error(const char* fmt, ...) {
   char buf[2048];
   va_list ap;
@@ -106,6 +111,7 @@ uint16_t float_to_half_bits(float f) {
 
 extern "C" {
 int scn_version(void) { return 10000; }
+size_t scn_device_bytes_in_use(void) { return scn::device_bytes_counter().load(); }
 const char* scn_last_error(void) { return scn::g_last_error.c_str(); }
 void scn_set_log_level(int level) { scn::g_level = level; }
 int scn_get_log_level(void) { return scn::g_level; }

@@ -1,6 +1,8 @@
 // Shared host-side helpers of libscn_hip: logging, error state, HIP call checking, device buffers.
 #pragma once
 
+#include <atomic>
+
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
@@ -74,6 +76,9 @@ struct HostBuf {
   }
 };
 
+// device bytes currently held by DevBuf objects of this process (scn_device_bytes_in_use)
+std::atomic<size_t>& device_bytes_counter();
+
 struct DevBuf {
   void* p = nullptr;
   size_t bytes = 0;
@@ -105,10 +110,14 @@ struct DevBuf {
       return false;
     }
     bytes = n;
+    device_bytes_counter() += n;
     return true;
   }
   void release() {
-    if (p) (void)hipFree(p);
+    if (p) {
+      (void)hipFree(p);
+      device_bytes_counter() -= bytes;
+    }
     p = nullptr;
     bytes = 0;
   }

@@ -403,14 +403,8 @@ constexpr int conv_lds_min_waves(int chunks, int mt, int waves) {
   return conv_lds_three_groups(chunks, mt, waves) ? 6 : (mt >= 2 && waves <= 4) ? 2 : waves <= 8 ? 4 : 3;
 }
 
-// AHEAD = iterations between the issue of an iteration's gathers / weight slab and their use.  1: one stage per
-// wave and two slab buffers, which is what fits the LDS of full CUs, and the only value the dispatch below
-// instantiates.  2: three of each, meant for launches of few rows (at most four 32-row tiles per CU).
-// NOT DISPATCHED: its first run on the GPU ended in a memory fault whose cause has not been found by reading
-// the code and its assembly; it must not be instantiated before it is.  (Later measurements with loads issued
-// earlier in the one-stage schedule found that neither gathers nor slabs are late, so it may not pay either.)
-template <int EL, int CHUNKS, int MT, int WAVES, int AHEAD = 1>
-__global__ __launch_bounds__(64 * WAVES, AHEAD > 1 ? 2 : conv_lds_min_waves(CHUNKS, MT, WAVES)) void k_conv_lds(const ConvArgs a) {
+template <int EL, int CHUNKS, int MT, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) void k_conv_lds(const ConvArgs a) {
   using Acc = typename Mma32<EL>::Acc;
   using Acc4 = typename Mma32<EL>::Acc4;
   constexpr int THREADS = 64 * WAVES;
@@ -426,12 +420,9 @@ __global__ __launch_bounds__(64 * WAVES, AHEAD > 1 ? 2 : conv_lds_min_waves(CHUN
   constexpr bool IDX4 = G >= 8;                  // 16-byte index loads (all 64 lanes busy; measured slower for G = 2, equal for 4)
   constexpr int IDXI = IDX4 ? 1 : IDXE;          // index loads per wave and iteration
   constexpr int R = 32 * WAVES;                  // output rows per workgroup
-  constexpr int NBUF = AHEAD + 1;                // slab buffers, and stages of gathered rows per wave
-  constexpr int NST = AHEAD > 1 ? NBUF : 1;
-  __shared__ v4i lds[NBUF][SLAB];
-  __shared__ v4i ring[WAVES][NST][256];
-  constexpr int DEPTH = AHEAD > 1 ? 4 : ((MT == 1 && CHUNKS <= 2) || conv_lds_three_groups(CHUNKS, MT, WAVES)) ? 2 : 4;   // index ring stages (LDS is what limits the narrow layers' occupancy)
-  static_assert(AHEAD >= 1 && AHEAD < DEPTH, "the index ring must reach past the gathers in flight");
+  __shared__ v4i lds[2][SLAB];                   // weight slabs of iterations i and i+1
+  __shared__ v4i ring[WAVES][1][256];            // one stage of gathered rows per wave
+  constexpr int DEPTH = ((MT == 1 && CHUNKS <= 2) || conv_lds_three_groups(CHUNKS, MT, WAVES)) ? 2 : 4;   // index ring stages (LDS is what limits the narrow layers' occupancy)
   __shared__ int32_t iring[DEPTH][WAVES][64 * IDXE];
   __shared__ v4i spare[NL % WAVES ? 64 : 1];
   const int tid = threadIdx.x;
@@ -574,7 +565,7 @@ __global__ __launch_bounds__(64 * WAVES, AHEAD > 1 ? 2 : conv_lds_min_waves(CHUN
   }
   // the 4 * MT MFMAs of an iteration: A fragments from the slab at LDS address la, B fragments bf[]
   auto multiply = [&](const uint32_t la, const v4i (&bf)[4]) {
-    if constexpr (AHEAD == 1 && WAVES >= 8 && ((MT >= 4 && conv_lds_min_waves(CHUNKS, MT, WAVES) >= 4) || conv_lds_three_groups(CHUNKS, MT, WAVES))) {
+    if constexpr (WAVES >= 8 && ((MT >= 4 && conv_lds_min_waves(CHUNKS, MT, WAVES) >= 4) || conv_lds_three_groups(CHUNKS, MT, WAVES))) {
       // 64 accumulator registers leave room for one set of fragments under the 128-register budget of
       // four waves per SIMD (a spill would also put scratch loads into the memory counter and break the
       // counts below); the other three waves of the SIMD cover the LDS latency instead.  (Workgroups of 2 or 4
@@ -612,7 +603,7 @@ __global__ __launch_bounds__(64 * WAVES, AHEAD > 1 ? 2 : conv_lds_min_waves(CHUN
   // the offsets that leave it, tiles next to empty space: a third to a half of all (tile, offset)
   // combinations of a synthetic frame, a tenth of a real one's) skips that iteration's operand reads and
   // MFMAs -- they would add zeros -- and, where the waits below can follow it, its gathers.
-  if constexpr (AHEAD == 1) {
+  {
     // prologue: indices of iterations 0 .. DEPTH-1, slab 0, then the gathers of iteration 0
     SCN_INDEX(0);
     SCN_INDEX(1);
@@ -658,52 +649,6 @@ __global__ __launch_bounds__(64 * WAVES, AHEAD > 1 ? 2 : conv_lds_min_waves(CHUN
       work = work_next;
       // every wave has read slab it (its fragments are in registers) and written its part of slab it+1
       asm volatile("s_barrier" ::: "memory");
-    }
-  } else {
-    // Loads of one iteration, in issue order: S (WPT), I (IDXI) at its top, G (4) in its middle; the gathers
-    // are issued for every iteration here (empty ones fetch the row of zeros) so that the counts hold.
-    constexpr int PER_IT = WPT + IDXI + 4;
-    // prologue: indices 0 .. DEPTH-1, slabs and gathers 0 .. AHEAD-1, everything landed
-    SCN_INDEX(0);
-    SCN_INDEX(1);
-    SCN_INDEX(2);
-    SCN_INDEX(3);
-#pragma unroll
-    for (int j = 0; j < AHEAD; ++j) SCN_SLAB(j, j);
-    SCN_WAIT_VM((DEPTH - AHEAD) * IDXI + AHEAD * WPT);  // I(0) .. I(AHEAD-1) have landed
-    uint32_t workbits = 0;  // wave-uniform; bit j: iteration it + j has at least one neighbour row
-#pragma unroll
-    for (int j = 0; j < AHEAD; ++j) {
-      int32_t gi[4];
-      SCN_READ_INDEX(j, gi);
-      if (__builtin_amdgcn_ballot_w64((gi[0] & gi[1] & gi[2] & gi[3]) >= 0) != 0) workbits |= 1u << j;
-      SCN_GATHER(j, gi, j);
-    }
-    SCN_WAIT_VM(0);
-    asm volatile("s_barrier" ::: "memory");
-
-    uint32_t rbuf = 0;  // it % NBUF: slab buffer and stage of the current iteration
-    for (int it = 0; it < iters; ++it) {
-      const uint32_t wbuf = rbuf == 0 ? (uint32_t)AHEAD : rbuf - 1;  // (it + AHEAD) % NBUF: read last in iteration it-1
-      SCN_SLAB(it + AHEAD, wbuf);
-      SCN_INDEX(it + DEPTH);
-      // G(it) has landed: younger are S and I of this iteration and everything of iterations it-AHEAD+1 .. it-1
-      SCN_WAIT_VM((AHEAD - 1) * PER_IT + WPT + IDXI);
-      const bool work = workbits & 1u;
-      v4i bf[4];
-      int32_t gi[4];
-      if (work) SCN_READ_B(rbuf, bf);
-      // waits for the index reads and, LDS returning in order, for the B reads of this and earlier iterations
-      SCN_READ_INDEX((it + AHEAD) & (DEPTH - 1), gi);
-      workbits >>= 1;
-      if (__builtin_amdgcn_ballot_w64((gi[0] & gi[1] & gi[2] & gi[3]) >= 0) != 0) workbits |= 1u << (AHEAD - 1);
-      SCN_GATHER(it + AHEAD, gi, wbuf);
-      if (work) multiply(lds_a_addr + rbuf * (uint32_t)(SLAB * 16), bf);
-      // this wave's part of S(it+1) has landed: younger are I and G of the iteration that issued it and
-      // everything of the AHEAD-1 iterations since
-      SCN_WAIT_VM(IDXI + 4 + (AHEAD - 1) * PER_IT);
-      asm volatile("s_barrier" ::: "memory");
-      rbuf = rbuf == (uint32_t)AHEAD ? 0u : rbuf + 1;
     }
   }
 #undef SCN_READ_B
@@ -1074,12 +1019,11 @@ static void launch_conv_rows(const ConvArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL((k_conv_rows<EL, CHUNKS, MT, NT>), dim3(blocks), dim3(256), 0, stream, a);
 }
 
-template <int EL, int CHUNKS, int MT, int WAVES, int AHEAD = 1>
+template <int EL, int CHUNKS, int MT, int WAVES>
 static void launch_conv_lds(const ConvArgs& a, hipStream_t stream) {
-  static_assert(AHEAD == 1, "the deeper load pipeline faulted on the GPU and is switched off");
   constexpr uint32_t R = 32 * WAVES;
   const uint32_t blocks = 8 * ceil_div(ceil_div(a.n_bound, R), 8);  // see xcd_tile()
-  hipLaunchKernelGGL((k_conv_lds<EL, CHUNKS, MT, WAVES, AHEAD>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
+  hipLaunchKernelGGL((k_conv_lds<EL, CHUNKS, MT, WAVES>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
 }
 
 // Workgroup size of the 128-channel kernel.  A layer of a lidar backbone's deep stages is about one

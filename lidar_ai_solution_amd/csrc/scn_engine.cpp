@@ -190,6 +190,7 @@ struct scn_engine {
   DevBuf amax_buf;                     // collect_amax: one 16-byte slot per tensor
   bool dense_map_built = false;        // the step about to run had its row map built on the auxiliary stream
   std::vector<DevBuf> dense_maps;      // per step: cell -> row map of a ScatterDense whose layout allows the dense-major pass
+  std::vector<DevBuf> arena;           // storage shared by sparse tensors whose lifetimes do not overlap
   std::map<std::string, int> tensor_by_name;
   // input binding
   const void* in_feat = nullptr;
@@ -875,6 +876,65 @@ static int allocate_runtime(scn_engine& e) {
     }
   }
   const bool keep_all = (e.flags & SCN_BUILD_KEEP_ALL) != 0;
+  // Lifetime of every tensor in step order (the feature kernels run in that order on one stream, with or without
+  // the auxiliary stream): from the step that writes it to the last step that reads it.  Sparse tensors whose
+  // lifetimes do not overlap share storage; a tensor written by a step never shares with one that step reads.
+  // Graph outputs and everything in keep-all engines own their storage.
+  const int never = 1 << 30;
+  std::vector<int> born(e.tensors.size(), never), dies(e.tensors.size(), -1);
+  for (size_t si = 0; si < e.steps.size(); ++si) {
+    const Step& st = e.steps[si];
+    for (int t : {st.t_in, st.t_in2, st.t_conv_in})
+      if (t >= 0 && t < (int)e.tensors.size()) dies[t] = std::max(dies[t], (int)si);
+    if (st.t_out >= 0 && st.t_out < (int)e.tensors.size()) {
+      born[st.t_out] = std::min(born[st.t_out], (int)si);
+      dies[st.t_out] = std::max(dies[st.t_out], (int)si);
+    }
+  }
+  for (int o : e.outputs) dies[o] = never;
+  struct Shared {
+    size_t bytes;
+    int busy_until;
+  };
+  std::vector<Shared> pool;
+  std::vector<int> slot_of(e.tensors.size(), -1);
+  {
+    std::vector<int> order;
+    for (size_t t = 0; t < e.tensors.size(); ++t) {
+      const RtTensor& x = e.tensors[t];
+      if (!x.materialised || (int)t == e.inputs[0] || x.dense || keep_all || born[t] == never || dies[t] == never) continue;
+      order.push_back((int)t);
+    }
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return born[a] < born[b]; });
+    for (int t : order) {
+      const RtTensor& x = e.tensors[t];
+      const size_t bytes = ((size_t)e.coords[x.coord].cap * x.ld * (x.dtype == SCN_DTYPE_INT8 ? 1 : 2) + 255) & ~(size_t)255;
+      int best = -1;
+      for (size_t k = 0; k < pool.size(); ++k)   // the free block that is closest in size
+        if (pool[k].busy_until < born[t]) {
+          if (best < 0) best = (int)k;
+          else {
+            const bool fits = pool[k].bytes >= bytes, best_fits = pool[best].bytes >= bytes;
+            if ((fits && !best_fits) || (fits == best_fits && (fits ? pool[k].bytes < pool[best].bytes : pool[k].bytes > pool[best].bytes)))
+              best = (int)k;
+          }
+        }
+      if (best < 0) {
+        pool.push_back(Shared{bytes, dies[t]});
+        best = (int)pool.size() - 1;
+      } else {
+        pool[best].bytes = std::max(pool[best].bytes, bytes);
+        pool[best].busy_until = dies[t];
+      }
+      slot_of[t] = best;
+    }
+  }
+  if (e.arena.size() < pool.size()) e.arena.resize(pool.size());
+  for (size_t k = 0; k < pool.size(); ++k)
+    if (e.arena[k].bytes < pool[k].bytes) {
+      if (!e.arena[k].alloc(pool[k].bytes)) return SCN_ERR_HIP;
+      SCN_HIP(hipMemset(e.arena[k].p, 0, pool[k].bytes));
+    }
   for (size_t t = 0; t < e.tensors.size(); ++t) {
     RtTensor& x = e.tensors[t];
     if (!x.materialised || (int)t == e.inputs[0]) continue;
@@ -885,6 +945,11 @@ static int allocate_runtime(scn_engine& e) {
       const size_t dbytes = (numel * (x.dtype == SCN_DTYPE_INT8 ? 1 : 2) + 15) & ~(size_t)15;
       if (x.buf.bytes < dbytes && !x.buf.alloc(dbytes)) return SCN_ERR_HIP;
       x.data = x.buf.p;
+      continue;
+    }
+    if (slot_of[t] >= 0) {
+      x.buf.release();
+      x.data = e.arena[slot_of[t]].p;
       continue;
     }
     const size_t rows = e.coords[x.coord].cap;

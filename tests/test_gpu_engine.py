@@ -705,3 +705,31 @@ def test_inverted_graph_on_device_gives_the_same_bev(bevfusion_input):
     _run_engine(eng_i, feats, export.invert_indices(idx), GRID_XYZ[::-1])
     got_i = eng_i.output(0).torch().cpu().numpy()
     assert got_i.shape == want.shape and np.array_equal(got_i.view(np.uint16), want.view(np.uint16))
+
+
+def test_device_memory_at_the_reference_defaults(centerpoint_input):
+    """Sparse tensors whose lifetimes do not overlap share storage.  At the reference's defaults (output_bound
+    150,000) the int8 CenterPoint-shaped engine holds less device memory than the reference publishes for its own
+    (422 / 426 MB, libraries/3DSparseConvolution/README.md:36-40), and gives the bits of a keep-all engine, which
+    shares nothing."""
+    feats, idx = centerpoint_input
+    L = capi.lib()
+    g16, tags = graphs.centerpoint_scn(seed=0, output_bound=150000)
+    amax = _oracle_calibration(g16, feats, idx, GRID_ZYX)
+    g8, tags8 = graphs.centerpoint_scn(seed=0, output_bound=150000)
+    graphs.apply_int8_plan(g8, tags8, amax, "centerpoint")
+    torch.cuda.synchronize()
+    for prec, graph in (("int8", g8), ("fp16", g16)):
+        before = L.scn_device_bytes_in_use()
+        eng = Engine.from_graph(graph, prec, with_auxiliary_stream=True)
+        _run_engine(eng, feats, idx, GRID_ZYX)
+        used = L.scn_device_bytes_in_use() - before
+        note(f"{prec} engine at output_bound 150,000: {used / 1e6:.1f} MB of device memory")
+        assert 0 < used <= 426e6, used
+        got = eng.output(0).torch().clone()
+        keep = Engine.from_graph(graph, prec, keep_all=True)
+        _run_engine(keep, feats, idx, GRID_ZYX)
+        assert torch.equal(keep.output(0).torch().view(torch.int16), got.view(torch.int16))
+        keep.close()
+        eng.close()
+        assert L.scn_device_bytes_in_use() == before
