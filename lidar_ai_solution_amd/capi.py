@@ -46,7 +46,7 @@ class ConvIO(C.Structure):
                 ("out_dynamic_range", C.c_float), ("out_dev", vp), ("out_ld", u32), ("acc_dev", vp), ("res_dev", vp),
                 ("res_dtype", C.c_int), ("res_dynamic_range", C.c_float), ("res_ld", u32), ("mid_dtype", C.c_int),
                 ("mid_dynamic_range", C.c_float), ("a_requant_range", C.c_float), ("b_requant_range", C.c_float),
-                ("relu_after_add", C.c_int)]
+                ("relu_after_add", C.c_int), ("fixed_launch_points", u32)]
 
 
 class TensorView(C.Structure):

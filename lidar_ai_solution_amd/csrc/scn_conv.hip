@@ -197,6 +197,11 @@ int conv_forward(const ConvWeights& w, const int32_t* nbr, uint32_t nbr_ld, cons
   if (w.precision == SCN_PRECISION_INT8)
     SCN_REQUIRE(io.x_dynamic_range > 0.f, SCN_ERR_INVALID, "conv: int8 input needs x_dynamic_range > 0");
   if (n_hint == 0 || n_hint > n_bound) n_hint = n_bound;
+  // fixed_launch_points (engine.hpp:107,150; src/infer.cpp:380-398): 0 sizes the grid for the bound, as a caller
+  // that knows nothing about its inputs must; otherwise for that many rows or for what the previous forward had,
+  // whichever is more
+  a.launch_rows = io.fixed_launch_points ? std::min(n_bound, std::max(io.fixed_launch_points, n_hint)) : n_bound;
+  if (a.launch_rows == 0) a.launch_rows = 1;
   const bool ok = w.precision == SCN_PRECISION_INT8 ? conv_dispatch_int8(w, n_hint, a, stream)
                                                     : conv_dispatch_fp16(w, n_hint, a, stream);
   SCN_REQUIRE(ok, SCN_ERR_UNSUPPORTED, "conv: no kernel for Cin=%d Cout=%d (chunks %d, m-tiles %d)", w.cin, w.cout,

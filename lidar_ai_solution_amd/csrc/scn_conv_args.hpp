@@ -13,6 +13,12 @@ struct ConvArgs {
   int kvol;
   const uint32_t* n_out_dev;
   uint32_t n_bound;
+  // rows the persistent grid of the tile-plan kernel is sized for, 1 .. n_bound: the larger of the caller's
+  // fixed_launch_points and the row count of the previous forward.  Never a limit: its waves loop over all tiles.
+  // (The LDS-staged kernels launch one workgroup per tile of the bound; workgroups beyond the count leave at once.
+  // A loop over tiles in those kernels was built and measured: the compiler then spills 100 .. 680 bytes of registers
+  // per lane and every layer takes 1.3 .. 2.4 times as long, while the surplus workgroups it saves cost under 1 us.)
+  uint32_t launch_rows;
   const uint4* wfrag;
   int steps;
   const float* wscale;

@@ -976,7 +976,8 @@ template <int EL, int CHUNKS, int MT>
 static void launch_conv_tile(const ConvArgs& a, uint32_t n_hint, hipStream_t stream) {
   // as many workgroups of 8 waves as fit the GPU at once (two or four per CU); fewer when the expected rows
   // are fewer than that many tiles
-  const uint32_t tiles = ceil_div(n_hint ? n_hint : a.n_bound, 32u);
+  (void)n_hint;
+  const uint32_t tiles = ceil_div(a.launch_rows, 32u);
   const uint32_t resident = 256u * (conv_tile_min_waves(CHUNKS, MT) / 2);
   uint32_t blocks = ceil_div(tiles, 8u);
   blocks = blocks < 1 ? 1 : blocks > resident ? resident : blocks;

@@ -54,6 +54,7 @@ struct NodeDesc {
   bool subm = false;
   bool inverse = false;
   uint32_t max_out = 150000;
+  uint32_t fixed_launch_points = 0;
   std::string rulebook;
   int precision = SCN_PRECISION_FP16, out_precision = SCN_PRECISION_FP16;
   // add
@@ -1105,6 +1106,7 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
       io.out_dev = o.data;
       io.out_ld = o.ld;
       io.acc_dev = o.acc.p;
+      io.fixed_launch_points = e.nodes[st.node].fixed_launch_points;
       if (st.fused_add) {
         const RtTensor& r = e.tensors[st.t_in2];
         io.res_dev = r.data;
@@ -1373,7 +1375,6 @@ int scn_builder_push_sparse_conv(scn_builder* b, const char* name, int x, const 
                                  const int dilation[3], float input_dynamic_range, int submanifold,
                                  uint32_t max_output_points, uint32_t fixed_launch_points, const char* rulebook,
                                  int precision, int output_precision, const char* output_name, int inverse) {
-  (void)fixed_launch_points;  // launch sizes always come from host-side bounds; nothing to fix
   if (!b || !b->valid_tensor(x) || !weight || !weight_shape || !kernel_size) {
     set_error("push_sparse_conv(%s): invalid arguments", name ? name : "");
     return -1;
@@ -1431,6 +1432,7 @@ int scn_builder_push_sparse_conv(scn_builder* b, const char* name, int x, const 
   n.subm = submanifold != 0;
   n.inverse = inverse != 0;
   n.max_out = max_output_points ? max_output_points : 150000;
+  n.fixed_launch_points = fixed_launch_points;
   n.rulebook = rulebook ? rulebook : "";
   n.precision = precision;
   n.out_precision = output_precision;

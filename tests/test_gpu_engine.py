@@ -733,3 +733,47 @@ def test_device_memory_at_the_reference_defaults(centerpoint_input):
         keep.close()
         eng.close()
         assert L.scn_device_bytes_in_use() == before
+
+
+def test_launch_configuration_chosen_for_a_small_frame_serves_a_large_one(cp_models, centerpoint_input):
+    """Launch configurations (workgroup heights, the persistent grid of the tile-plan kernel, which honours
+    fixed_launch_points: engine.hpp:107,150, src/infer.cpp:380-398) are chosen from the previous forward's row counts
+    and never limit what is computed.  A forward on 3,000 rows followed by one on all 79,745 -- direct, and as
+    replays of a graph captured while the small frame was the last one seen -- gives the bits of a fresh engine,
+    with and without sortmask."""
+    feats, idx = centerpoint_input
+    _, g8 = cp_models
+    n_full = feats.shape[0]
+    fresh = Engine.from_graph(g8, "int8")
+    _run_engine(fresh, feats, idx, GRID_ZYX)
+    want = fresh.output(0).torch().clone()
+    f, i = to_dev(feats), to_dev(idx)
+    cnt = torch.tensor([3000], dtype=torch.int32, device=DEV)
+    for aux in (False, True):
+        note(f"small frame, then the full one on launches chosen for the small one (auxiliary stream / sortmask {aux})")
+        eng = Engine.from_graph(g8, "int8", with_auxiliary_stream=aux, sortmask=aux)
+        eng.set_input(f, i, GRID_ZYX)
+        eng.set_dds_num_of_points_pointer(cnt)
+        cnt.fill_(3000)
+        eng.forward()
+        torch.cuda.synchronize()          # the host now knows the small row counts
+        small = eng.output(0).torch().clone()
+        cnt.fill_(n_full)
+        eng.forward()                     # launched for ~10,000 rows per layer, 79,745 arrive
+        torch.cuda.synchronize()
+        assert torch.equal(eng.output(0).torch().view(torch.int16), want.view(torch.int16))
+        note("graph captured after the small frame, replayed on the full one and on the small one")
+        cnt.fill_(3000)
+        eng.forward()
+        torch.cuda.synchronize()
+        st = torch.cuda.Stream()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=st):
+            eng.forward()
+        torch.cuda.synchronize()
+        for n_now, expect in ((n_full, want), (3000, small), (n_full, want)):
+            cnt.fill_(n_now)
+            assert np.isfinite(torch.randn(1 << 18, device=DEV).sum().item())
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(eng.output(0).torch().view(torch.int16), expect.view(torch.int16)), n_now
