@@ -374,6 +374,47 @@ __global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_
   }
 }
 
+// Strided rulebooks build their table from the input side: an output row has 27 candidate inputs of which a
+// lidar frame fills 1 .. 5, an input row has at most 27 outputs that all exist.  Two kernels: every entry of the
+// rows in use becomes -1 (16-byte stores; rows up to the next multiple of 32, see Rulebook::nbr), then one thread
+// per (input row, k0, k1) walks k2, finds the output cell o = (i + pad - k dil) / stride where that division is
+// exact, its row by bitmap rank, and enters itself.  For a fixed offset an output has one input cell, so entries
+// have one writer unless the caller's coordinates repeat; the smallest row then wins, as in the coordinate hash.
+__global__ __launch_bounds__(256) void k_clear_table(int32_t* nbr, uint32_t ld, const uint32_t* n_out_dev,
+                                                     uint32_t n_bound, uint32_t* n_host) {
+  const uint32_t n = eff_n(n_out_dev, n_bound);
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0 && n_host) *n_host = n;
+  const uint32_t j = (blockIdx.x * 256 + threadIdx.x) * 4;
+  if (j >= ((n + 31u) & ~31u)) return;
+  *reinterpret_cast<int4*>(nbr + (size_t)blockIdx.y * ld + j) = make_int4(-1, -1, -1, -1);
+}
+
+__global__ __launch_bounds__(256) void k_scatter_nbr(const int4* __restrict__ in_coords, const uint32_t* n_in_dev,
+                                                     uint32_t n_in_bound, GeomDev g, CoordLookup out_lk, int32_t* nbr,
+                                                     uint32_t ld) {
+  const uint32_t n = eff_n(n_in_dev, n_in_bound);
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int4 c = in_coords[i];
+  if (c.x != 0 || c.y < 0 || c.y >= g.gi[0] || c.z < 0 || c.z >= g.gi[1] || c.w < 0 || c.w >= g.gi[2]) return;
+  const int k01 = blockIdx.y;
+  const int k0 = k01 / g.ks[1], k1 = k01 - k0 * g.ks[1];
+  const int t0 = c.y + g.pd[0] - k0 * g.dl[0], t1 = c.z + g.pd[1] - k1 * g.dl[1];
+  if (t0 < 0 || t1 < 0) return;
+  const int o0 = t0 / g.st[0], o1 = t1 / g.st[1];
+  if (o0 * g.st[0] != t0 || o1 * g.st[1] != t1 || o0 >= g.go[0] || o1 >= g.go[1]) return;
+  const uint32_t line = ((uint32_t)o0 * (uint32_t)g.go[1] + (uint32_t)o1) * (uint32_t)g.go[2];
+  for (int k2 = 0; k2 < g.ks[2]; ++k2) {
+    const int t2 = c.w + g.pd[2] - k2 * g.dl[2];
+    if (t2 < 0) continue;
+    const int o2 = t2 / g.st[2];
+    if (o2 * g.st[2] != t2 || o2 >= g.go[2]) continue;
+    const int32_t o = coord_row(out_lk, line + (uint32_t)o2);
+    if (o < 0) continue;   // (an output beyond the row bound)
+    atomicMin(reinterpret_cast<uint32_t*>(nbr) + (size_t)(k01 * g.ks[2] + k2) * ld + (uint32_t)o, i);
+  }
+}
+
 // Marks every output cell reached by an input row through some kernel offset.  One thread per
 // input row; per axis the (at most K) reachable output coordinates are found first, then their
 // combinations are marked -- the bits of one output line that fall into the same word in one
@@ -627,8 +668,32 @@ int Rulebook::build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev
                        blocksum.as<uint32_t>(), og, n_bound_out, (int4*)out_idx.p, prefix.as<uint32_t>(), raw, cnt);
   }
   SCN_HIP(hipGetLastError());
-  rc = launch_build_nbr(*this, out_indices, cnt, n_bound_out, false, nullptr, stream);
-  if (rc) return rc;
+  // The table: from the output side (every output row looks up its candidate inputs) or from the input side (see
+  // k_scatter_nbr).  The first costs rows_out x volume look-ups, the second a clear of as many entries plus two
+  // dependent loads and an atomic per pair: measured on a 123 k -> 322 k-row stage (1.3 pairs per output) 37 -> 21 us
+  // from the input side, on 322 k -> 215 k rows (4.7 pairs per output) 13 us slower.  So: the input side when the
+  // outputs expected (the previous forward's count) are at least twice the inputs.  SCN_RULEBOOK_TABLE=gather /
+  // scatter forces one.
+  static const int forced = [] {
+    const char* e = getenv("SCN_RULEBOOK_TABLE");
+    return !e ? 0 : !strcmp(e, "gather") ? 1 : !strcmp(e, "scatter") ? 2 : 0;
+  }();
+  const bool gather_build = forced == 1 || (forced == 0 && (uint64_t)n_out_hint() < 2ull * n);
+  if (gather_build) {
+    rc = launch_build_nbr(*this, out_indices, cnt, n_bound_out, false, nullptr, stream);
+    if (rc) return rc;
+  } else {
+    const uint32_t pos = (n_bound_out + 31u) & ~31u;
+    if (pos)
+      hipLaunchKernelGGL(k_clear_table, dim3(ceil_div(pos / 4, 256), geom.kvol), dim3(256), 0, stream, nbr.as<int32_t>(), ld,
+                         cnt, n_bound_out, host_count.as<uint32_t>());
+    else
+      *host_count.as<uint32_t>() = 0;
+    if (n && pos)
+      hipLaunchKernelGGL(k_scatter_nbr, dim3(ceil_div(n, 256), geom.ks[0] * geom.ks[1]), dim3(256), 0, stream,
+                         (const int4*)idx, n_dev, n, gd, out_lookup(), nbr.as<int32_t>(), ld);
+    SCN_HIP(hipGetLastError());
+  }
   built = true;
   return SCN_OK;
 }
