@@ -364,9 +364,16 @@ def main():
     # which roof bounds the kernel: its algorithmic intensity against the machine balance (ops per HBM byte)
     intensity = dom_ops / dom_bytes
     ridge = mfma_peak * 1e12 / (HBM_PEAK_GBS * 1e9)
-    kernel = (f"k_conv_lds {args.precision} Cin={dom_key[0]} Cout={dom_key[1]} {'subm' if dom_key[2] else 'strided'} "
-              f"k={'x'.join(map(str, dom_key[3]))}")
-    traffic, traffic_from = measured_traffic(args.precision, dom_key, nvox, args.output_bound)
+    # under sortmask the narrow layers (input rows of at most 64 bytes, at most 64 output channels, kernel volume
+    # at most 31, all weights within 60 KB of LDS) run the tile-plan kernel
+    row_bytes = -(-dom_key[0] * (1 if args.precision == "int8" else 2) // 16) * 16
+    kvol, mt32 = int(np.prod(dom_key[3])), -(-dom_key[1] // 32)
+    on_plan = (args.sortmask and kvol <= 31 and mt32 <= 2 and row_bytes in (16, 32, 64)
+               and -(-kvol * (row_bytes // 16) // 2) * mt32 * 1024 + 512 <= 60 * 1024)
+    kernel = (f"{'k_conv_tile' if on_plan else 'k_conv_lds'} {args.precision} Cin={dom_key[0]} Cout={dom_key[1]} "
+              f"{'subm' if dom_key[2] else 'strided'} k={'x'.join(map(str, dom_key[3]))}")
+    traffic, traffic_from = (None, None) if args.sortmask else measured_traffic(args.precision, dom_key, nvox,
+                                                                                args.output_bound)
     # rows of every strided convolution's output: kept (what the layers after it run on) and before the
     # output_bound cut; equal unless the bound truncates
     stage_rows = []
