@@ -35,6 +35,27 @@ def test_half_conversion_matches_numpy():
 
 
 def test_hash_is_64bit_murmur_finaliser():
+    # The hash only places keys in the reference's open-addressing table; no output depends on it, so this is a guard
+    # on the C restatement (64-bit evaluation, libraries/3DSparseConvolution/src/voxelization.cu:41-48), not a parity pin.
+    # What the structure fixes without re-typing it: xor-shifts and odd multiplications are invertible modulo 2^64, so
+    # the function is a bijection and undoing the steps with the modular inverses must give the key back.
+    M = (1 << 64) - 1
+    def unshift(v, s):
+        r = v
+        for _ in range(64 // s + 1):
+            r = v ^ (r >> s)
+        return r
+    def inverse(h):
+        h = unshift(h, 16)
+        h = (h * pow(0xC2B2AE35, -1, 1 << 64)) & M
+        h = unshift(h, 13)
+        h = (h * pow(0x85EBCA6B, -1, 1 << 64)) & M
+        return unshift(h, 16)
+    rng0 = np.random.default_rng(7)
+    keys = [int(v) for v in rng0.integers(0, 2 ** 32, 3000)]
+    assert all(inverse(O.hash64(k)) == k for k in keys)
+    assert len({O.hash64(k) for k in keys}) == len(set(keys))
+
     def py(k):
         M = (1 << 64) - 1
         k ^= k >> 16
