@@ -98,9 +98,12 @@ __device__ __forceinline__ bool coord_key(const int4 c, const Int3 g, uint32_t* 
 
 // filter (nullable): occupancy bitmap of the grid, set for every inserted coordinate; lookups test it
 // before probing the table (most neighbour lookups of a sparse tensor miss).
+// skip_if_zero (nullable): the "not in canonical order" flag of k_index_sorted_rows, which ran just before; while
+// it is 0 the rows need no hash and the whole grid leaves at once.
 __global__ __launch_bounds__(256) void k_hash_insert(uint64_t* slots, uint32_t mask, const int4* __restrict__ coords,
                                                      uint32_t n_bound, const uint32_t* n_dev, Int3 grid,
-                                                     uint32_t* n_eff_out, uint32_t* filter) {
+                                                     uint32_t* n_eff_out, uint32_t* filter,
+                                                     const uint32_t* skip_if_zero) {
   __shared__ uint32_t akeys[kAggSlots], avals[kAggSlots];
   const uint32_t n = eff_n(n_dev, n_bound);
   const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
@@ -108,6 +111,7 @@ __global__ __launch_bounds__(256) void k_hash_insert(uint64_t* slots, uint32_t m
     n_eff_out[0] = n;
     n_eff_out[1] = n;
   }
+  if (skip_if_zero && *skip_if_zero == 0) return;
   if (filter) agg_init(akeys, avals);
   uint32_t key;
   if (r < n && coord_key(coords[r], grid, &key)) {
@@ -115,6 +119,39 @@ __global__ __launch_bounds__(256) void k_hash_insert(uint64_t* slots, uint32_t m
     if (filter) agg_or(akeys, avals, filter, key >> 5, 1u << (key & 31));
   }
   if (filter) agg_flush(akeys, avals, filter);
+}
+
+// Rows in canonical order (strictly ascending linear index, every coordinate inside the grid): the first row of
+// every occupied 32-cell word ORs the bits of its run of rows (at most 32, consecutive) and writes the word and its
+// own row number with plain stores.  Any row that breaks the order raises *unsorted; what was written by then is
+// a subset of the true occupancy, which the hash insert that follows completes with its atomics.
+__global__ __launch_bounds__(256) void k_index_sorted_rows(const int4* __restrict__ coords, uint32_t n_bound,
+                                                           const uint32_t* n_dev, Int3 grid, uint32_t* bitmap,
+                                                           uint32_t* first_row, uint32_t* unsorted) {
+  const uint32_t n = eff_n(n_dev, n_bound);
+  const uint32_t r = blockIdx.x * 256 + threadIdx.x;
+  if (r >= n) return;
+  uint32_t key;
+  if (!coord_key(coords[r], grid, &key)) {
+    *unsorted = 1u;
+    return;
+  }
+  if (r > 0) {
+    uint32_t kp;
+    if (!coord_key(coords[r - 1], grid, &kp) || kp >= key) {
+      *unsorted = 1u;
+      return;
+    }
+    if ((kp >> 5) == (key >> 5)) return;  // not the first row of its word
+  }
+  uint32_t bits = 1u << (key & 31);
+  for (uint32_t j = r + 1; j < n && j < r + 32; ++j) {
+    uint32_t kj;
+    if (!coord_key(coords[j], grid, &kj) || (kj >> 5) != (key >> 5)) break;
+    bits |= 1u << (kj & 31);
+  }
+  bitmap[key >> 5] = bits;
+  first_row[key >> 5] = r;
 }
 
 __global__ void k_hash_query(const uint64_t* __restrict__ slots, uint32_t mask, const int4* __restrict__ coords,
@@ -146,8 +183,19 @@ bool CoordTable::alloc_filter(const int grid[3]) {
     return true;
   }
   const size_t words = (size_t)((cells + 31) / 32 + 3) & ~(size_t)3;
-  if (words > filter.bytes / 4 && !filter.alloc(words * 4)) return false;
+  if ((words + 4) > filter.bytes / 4 && !filter.alloc((words + 4) * 4)) return false;
   filter_words = words;
+  static const bool no_rank = [] {
+    const char* e = getenv("SCN_INPUT_INDEX");   // "hash": never try the canonical-order index (A/B measurements)
+    return e && !strcmp(e, "hash");
+  }();
+  if (!no_rank) {
+    if (words > first_row.bytes / 4 && !first_row.alloc(words * 4)) return false;
+    if (!sorted_hint.p) {
+      if (!sorted_hint.alloc(16)) return false;
+      *sorted_hint.as<uint32_t>() = 0;
+    }
+  }
   return true;
 }
 
@@ -169,15 +217,25 @@ int hash_build(const CoordTable& t, const int32_t* idx, uint32_t n, const uint32
     rc = fill_u32(t.slots(), 0xFFFFFFFFu, ((size_t)t.mask + 1) * 2, stream);
     if (rc) return rc;
     if (t.filter_words) {
-      rc = fill_u32(t.filter.p, 0u, t.filter_words, stream);
+      rc = fill_u32(t.filter.p, 0u, t.filter_fill_words(), stream);   // (with the order flag behind the words)
       if (rc) return rc;
     }
   }
-  const_cast<CoordTable&>(t).precleared_for = 0xFFFFFFFFu;
+  CoordTable& tm = const_cast<CoordTable&>(t);
+  tm.precleared_for = 0xFFFFFFFFu;
   Int3 g{{grid[0], grid[1], grid[2]}};
   const uint32_t blocks = n ? ceil_div(n, 256) : 1;
+  // the canonical-order index first, when the previous build found that order (or nothing is known yet, or it is
+  // time to look again); the hash insert then runs only if the order does not hold
+  tm.probed = t.filter_words && t.first_row.p && t.sorted_hint.p &&
+              (t.builds == 0 || *t.sorted_hint.as<uint32_t>() != 0 || t.builds % 16 == 0);
+  tm.builds++;
+  if (tm.probed)
+    hipLaunchKernelGGL(k_index_sorted_rows, dim3(blocks), dim3(256), 0, stream, (const int4*)idx, n, n_dev, g,
+                       t.filter.as<uint32_t>(), t.first_row.as<uint32_t>(), t.unsorted_flag());
   hipLaunchKernelGGL(k_hash_insert, dim3(blocks), dim3(256), 0, stream, t.slots(), t.mask,
-                     (const int4*)idx, n, n_dev, g, n_eff_out, t.filter_words ? t.filter.as<uint32_t>() : nullptr);
+                     (const int4*)idx, n, n_dev, g, n_eff_out, t.filter_words ? t.filter.as<uint32_t>() : nullptr,
+                     tm.probed ? (const uint32_t*)t.unsorted_flag() : (const uint32_t*)nullptr);
   SCN_HIP(hipGetLastError());
   return SCN_OK;
 }
@@ -339,12 +397,20 @@ __global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_
                                                    uint32_t* n_host) {
   const uint32_t n = eff_n(n_out_dev, n_bound);
   const uint32_t o = blockIdx.x * 256 + threadIdx.x;
+  // a hash table whose build found the rows in canonical order answers by rank
+  const bool by_rank = lk.unsorted != nullptr && *lk.unsorted == 0;
+  if (by_rank) {
+    lk.bitmap = lk.filter;
+    lk.prefix = lk.first_row;
+    lk.rank_cap = 0xFFFFFFFFu;
+  }
   if (o == 0 && blockIdx.y == 0) {
     if (n_publish) {
       n_publish[0] = n;
       n_publish[1] = n;
     }
     if (n_host) *n_host = n;  // pinned host word: the row count as a launch hint for the next forward
+    if (lk.sorted_hint_host) *lk.sorted_hint_host = by_rank ? 1u : 0u;
   }
   const int k01 = blockIdx.y;  // k0 * K1 + k1
   if (o >= n) {
@@ -522,6 +588,11 @@ CoordLookup CoordTable::lookup() const {
   lk.slots = slots();
   lk.mask = mask;
   lk.filter = filter_words ? filter.as<uint32_t>() : nullptr;
+  if (probed) {
+    lk.unsorted = unsorted_flag();
+    lk.first_row = first_row.as<uint32_t>();
+  }
+  lk.sorted_hint_host = sorted_hint.as<uint32_t>();   // (the consumer records 0 when the build did not look)
   return lk;
 }
 
@@ -933,7 +1004,7 @@ int scn_hash_build(uint64_t* table_dev, size_t capacity, const int32_t* indices_
   if (n) {
     hipLaunchKernelGGL(k_hash_insert, dim3(ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, table_dev,
                        (uint32_t)(capacity - 1), (const int4*)indices_dev, n, n_dev, g, (uint32_t*)nullptr,
-                       (uint32_t*)nullptr);
+                       (uint32_t*)nullptr, (const uint32_t*)nullptr);
     SCN_HIP(hipGetLastError());
   }
   return SCN_OK;

@@ -1020,7 +1020,7 @@ static int run_step(scn_engine& e, Step& st, hipStream_t stream) {
           const size_t words = hash_capacity_for(n) * 2;
           if (words <= t.cap * 2 && nj + (t.filter_words ? 2 : 1) <= kMaxFillJobs) {
             add(t.slots(), words, 0xFFFFFFFFu);
-            if (t.filter_words) add(t.filter.p, t.filter_words, 0u);
+            if (t.filter_words) add(t.filter.p, t.filter_fill_words(), 0u);
             t.precleared_for = n;
           }
         } else if (s2.kind == StepKind::RulebookSparse) {

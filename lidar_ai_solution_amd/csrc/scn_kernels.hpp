@@ -17,14 +17,32 @@ struct CoordLookup {
   const uint32_t* prefix = nullptr;
   uint32_t rank_cap = 0;  // ranks >= rank_cap were truncated away
   const uint32_t* filter = nullptr;  // hash lookups: occupancy bitmap tested before probing (nullable)
+  // Hash tables whose build also indexed the rows as a canonical-order tensor (see CoordTable): when *unsorted is 0
+  // the rows were strictly ascending in linear index, the filter is their occupancy bitmap and first_row[word] the row
+  // of the word's lowest set bit, so a look-up is a rank (two loads) and the hash table was not filled at all.
+  const uint32_t* unsorted = nullptr;
+  const uint32_t* first_row = nullptr;
+  uint32_t* sorted_hint_host = nullptr;  // pinned host word: 1 when the last build that has run found canonical order
 };
 
 struct CoordTable {
   DevBuf buf;
   size_t cap = 0;     // allocated slots, power of two
   uint32_t mask = 0;  // slots in use - 1 (power of two <= cap), set by the last build
-  DevBuf filter;             // occupancy bitmap of the grid (optional, see alloc_filter)
+  DevBuf filter;             // occupancy bitmap of the grid (optional, see alloc_filter); four more words follow it,
+                             // the first of which is the "rows are not in canonical order" flag of the last build
   size_t filter_words = 0;
+  // Canonical-order inputs (rows strictly ascending in linear voxel index: what a voxelizer that ranks cells emits)
+  // need no hash: one kernel without atomics writes each occupied word of the filter and the row of its first
+  // voxel, and look-ups become ranks.  The kernel also checks the order; when it does not hold, the hash insert
+  // that follows (and skips itself otherwise) fills table and filter as for any caller order.  Whether the check
+  // is launched at all follows the previous build's finding (a pinned host word), re-examined every 16th build.
+  DevBuf first_row;
+  HostBuf sorted_hint;
+  uint32_t builds = 0;
+  bool probed = false;       // the last build launched the canonical-order kernel
+  size_t filter_fill_words() const { return filter_words ? filter_words + 4 : 0; }
+  uint32_t* unsorted_flag() const { return filter.as<uint32_t>() + filter_words; }
   uint32_t precleared_for = 0xFFFFFFFFu;  // row count for which slots + filter were cleared by a batched fill
   bool alloc_for(uint32_t max_rows);
   bool alloc_filter(const int grid[3]);

@@ -135,6 +135,61 @@ def test_sparse_rulebook_truncation_empty_and_device_count():
     _check_pairs(s2, O.rulebook_subm(idx, grid, (3, 3, 3), (2, 2, 2)))
 
 
+def test_row_lookup_of_canonical_and_caller_order_inputs_on_one_rulebook():
+    """Rows in canonical order (strictly ascending linear index) are found by rank in an occupancy bitmap written
+    without atomics, any other order through the coordinate hash; which of the two a build tries first follows what
+    the previous build found.  One rulebook object sees both orders in turn (more than 16 builds, so that the periodic
+    second look happens too) and near-misses of the order: a swapped pair, a row outside the
+    grid, a device-side count that cuts the rows.  Every table must equal the oracle's."""
+    rng = np.random.default_rng(5)
+    grid = (7, 45, 70)
+    vol = int(np.prod(grid))
+    n = 2500
+
+    def coords(lin):
+        idx = np.zeros((lin.size, 4), np.int32)
+        idx[:, 3] = lin % grid[2]; idx[:, 2] = (lin // grid[2]) % grid[1]; idx[:, 1] = lin // (grid[2] * grid[1])
+        return idx
+
+    lin_sorted = np.sort(rng.choice(vol, n, replace=False))
+    cases = []
+    for i in range(18):
+        lin = np.sort(rng.choice(vol, n, replace=False))
+        if i % 3 == 2:
+            lin = rng.permutation(lin)
+        cases.append((f"build {i}: {'caller' if i % 3 == 2 else 'canonical'} order", coords(lin), n))
+    swapped = lin_sorted.copy(); swapped[[1200, 1201]] = swapped[[1201, 1200]]
+    cases.append(("one swapped pair", coords(swapped), n))
+    cases.append(("canonical again", coords(lin_sorted), n))
+    cases.append(("device-side count 1000 of canonical rows", coords(lin_sorted), 1000))
+    last_in_word = coords(lin_sorted[: n - 1])
+    cases.append(("one row fewer", last_in_word, n - 1))
+    sub = GpuRulebook(n, n, 27)
+    sp = GpuRulebook(n, n * 8, 27)
+    for label, idx, count in cases:
+        note("row lookup: " + label)
+        d_idx = to_dev(idx)
+        n_dev = None if count == idx.shape[0] else torch.tensor([count], dtype=torch.int32, device=DEV)
+        sub.build_subm(d_idx, idx.shape[0], grid, (3, 3, 3), n_dev=n_dev)
+        _check_pairs(sub, O.rulebook_subm(idx[:count], grid, (3, 3, 3)))
+        sp.build_sparse(d_idx, idx.shape[0], grid, (3, 3, 3), (2, 2, 2), (1, 1, 1), n_dev=n_dev)
+        ref = O.rulebook_sparse(idx[:count], grid, (3, 3, 3), (2, 2, 2), (1, 1, 1))
+        assert sp.n_out() == ref.n_out and np.array_equal(sp.out_indices(), ref.out_indices)
+        _check_pairs(sp, ref)
+    note("row lookup: one row outside the grid among canonical rows")
+    # (what such a row itself pairs with is not defined; every other row must see the tensor without it)
+    outside = coords(lin_sorted); outside[77, 3] = grid[2]
+    sub.build_subm(to_dev(outside), n, grid, (3, 3, 3))
+    pin, pout, offs = sub.pairs(27 * n)
+    ref = O.rulebook_subm(np.delete(outside, 77, axis=0), grid, (3, 3, 3))
+    shift = lambda r: r + (r >= 77)
+    for k in range(27):
+        got = {(int(a), int(b)) for a, b in zip(pin[offs[k]:offs[k + 1]], pout[offs[k]:offs[k + 1]]) if a != 77 and b != 77}
+        want = {(int(shift(a)), int(shift(b))) for a, b in zip(ref.pair_in[ref.offsets[k]:ref.offsets[k + 1]],
+                                                               ref.pair_out[ref.offsets[k]:ref.offsets[k + 1]])}
+        assert got == want, k
+
+
 # ----------------------------------------------------------------------------- convolution
 def _weights(rng, cout, ks, cin, std=0.02):
     w = (rng.standard_normal((cout, *ks, cin)) * std).astype(np.float16)
