@@ -26,13 +26,41 @@ def sources():
     return src
 
 
+# Kernels whose memory waits are counted by hand (s_waitcnt vmcnt(N) names which load has landed): a register spill
+# adds scratch loads to that counter behind the code's back, so a build in which one of them uses scratch memory fails.
+# The compiler reports every kernel's resources as remarks; they are read from the output of these translation units.
+NO_SCRATCH_KERNELS = ("k_conv_lds",)   # (k_conv_tile and k_conv_rows leave their waits to the compiler)
+RESOURCE_REMARKS = "-Rpass-analysis=kernel-resource-usage"
+
+
+def kernels_with_scratch(compiler_output: str):
+    """[(mangled kernel name, bytes per lane)] of the hand-counted kernels that the remarks report scratch for."""
+    found, name = [], None
+    for line in compiler_output.splitlines():
+        if "remark:" not in line:
+            continue
+        if "Function Name:" in line:
+            name = line.split("Function Name:", 1)[1].split("[", 1)[0].strip()
+        elif "ScratchSize [bytes/lane]:" in line and name is not None:
+            size = int(line.split("ScratchSize [bytes/lane]:", 1)[1].split("[", 1)[0].strip())
+            if size > 0 and any(k in name for k in NO_SCRATCH_KERNELS):
+                found.append((name, size))
+    return found
+
+
 def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    spilled = kernels_with_scratch(proc.stdout) if RESOURCE_REMARKS in cmd else []
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l and "kernel-resource-usage" not in l
+                    and not (RESOURCE_REMARKS in cmd and (l.lstrip().startswith(("|", "^")) or "__launch_bounds__" in l
+                                                          or l.startswith("In file included"))))
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed: " + " ".join(cmd) + "\n" + out)
+    if spilled:
+        raise RuntimeError("kernels with hand-counted memory waits use scratch memory (register spills):\n" +
+                           "\n".join(f"  {n}: {b} bytes per lane" for n, b in spilled))
     if verbose and out.strip():
         print(out)
 
@@ -63,7 +91,8 @@ def build(verbose: bool = False, jobs: int = 0, incremental: bool = False) -> st
         objs.append(obj)
         if incremental and not _stale(obj, src):
             continue
-        cmds.append(["hipcc", *compile_flags, "-I" + os.path.join(ROOT, "include"), "-c", src, "-o", obj])
+        remarks = [RESOURCE_REMARKS] if os.path.basename(src).startswith("scn_conv_") else []
+        cmds.append(["hipcc", *compile_flags, *remarks, "-I" + os.path.join(ROOT, "include"), "-c", src, "-o", obj])
     with ThreadPoolExecutor(max_workers=jobs_) as pool:
         list(pool.map(lambda c: _run(c, verbose), cmds))
     _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-fvisibility=hidden", "-no-hip-rt", *objs, "-o", LIB_PATH],

@@ -599,6 +599,31 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
     }
   };
 
+  // Residual tile of a fused Add (same element type as the output, see the epilogue): fetched into the wave's stage
+  // by the last iteration, once that iteration's B fragments are in registers, so that its latency passes behind the
+  // last MFMAs instead of in front of the epilogue.  Same placement as the epilogue's own staging: lane l of load q
+  // holds position l % 8 of tile row l / 8 + 8 q, i.e. chunk (l % 8) ^ (row % 8) of that row (first 128-byte pass).
+  // (Everything it needs is re-derived from the kernel arguments where it is used: a value kept across the loop
+  // costs a register, and these kernels have none to spare.)
+  // Not in the kernels compiled for 80 registers (three workgroups per CU) nor in the 8-wave kernels with 128 output
+  // channels (128 registers): there the few extra address registers of the last iteration spill, and spills are loads
+  // the counted waits do not know about.
+  constexpr bool RES_EARLY = !conv_lds_three_groups(CHUNKS, MT, WAVES) && !(MT >= 4 && WAVES == 8);
+#define SCN_RES_DMA() (RES_EARLY && a.res && a.res_vec16 && a.res_dtype == a.out_dtype && a.cout > 16 && a.out_vec16)
+#define SCN_RESIDUAL()                                                                          \
+  {                                                                                             \
+    const int res_esz = a.out_dtype == SCN_DTYPE_INT8 ? 1 : 2;                                  \
+    const int res_valid = ((a.cout + 15) & ~15) * res_esz;                                      \
+    _Pragma("unroll") for (int q = 0; q < 4; ++q) {                                             \
+      const int r_ = (lane >> 3) + 8 * q, c_ = (lane & 7) ^ (r_ & 7);                           \
+      const uint32_t grow_ = row0 + (uint32_t)r_;                                               \
+      const char* p_ = (grow_ < n && c_ * 16 < res_valid)                                       \
+                           ? a.res + (size_t)grow_ * a.res_ld * res_esz + c_ * 16               \
+                           : zrow + c_ * 16;                                                    \
+      __builtin_amdgcn_global_load_lds((gptr_t)p_, (lptr_t)&ring[wave][0][q * 64], 16, 0, 0);   \
+    }                                                                                           \
+  }
+
   // A wave whose 32 rows have no neighbour at any kernel offset of an iteration (rows of one z slice and
   // the offsets that leave it, tiles next to empty space: a third to a half of all (tile, offset)
   // combinations of a synthetic frame, a tenth of a real one's) skips that iteration's operand reads and
@@ -638,10 +663,15 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
       SCN_READ_INDEX((it + 1) & (DEPTH - 1), gi);
       // (iterations past the end read -1 everywhere)
       const bool work_next = __builtin_amdgcn_ballot_w64((gi[0] & gi[1] & gi[2] & gi[3]) >= 0) != 0;
-      if (work_next) SCN_GATHER(it + 1, gi, 0);
-      if (work) multiply(lds_a_addr + (uint32_t)(it & 1) * (SLAB * 16), bf);
-      // this wave's part of S(it+1) has landed (younger: G(it+1), when it was issued)
+      const bool res_now = it + 1 == iters && SCN_RES_DMA();   // (the last iteration has no next gathers: work_next is false)
       if (work_next) {
+        SCN_GATHER(it + 1, gi, 0);
+      } else if (res_now) {
+        SCN_RESIDUAL();
+      }
+      if (work) multiply(lds_a_addr + (uint32_t)(it & 1) * (SLAB * 16), bf);
+      // this wave's part of S(it+1) has landed (younger: G(it+1) or the residual tile, when issued)
+      if (work_next || res_now) {
         SCN_WAIT_VM(4);
       } else {
         SCN_WAIT_VM(0);
@@ -660,11 +690,14 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
 #undef SCN_SLAB
 #undef SCN_INDEX
 #undef SCN_GATHER
+#undef SCN_RESIDUAL
   // Epilogue.  Nothing in it may wait for global memory once per 4-channel piece (16 pieces per lane
   // for 128 channels, each a cache round trip): the per-channel constants are staged in LDS once per
   // workgroup, in the weight slab's space, and a residual tile is staged per wave like the output.
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stage still receives the gathers issued past the end
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stage still receives what the last iteration issued
   const int cout_pad = (a.cout + 15) & ~15;
+  const bool res_dma = SCN_RES_DMA();
+#undef SCN_RES_DMA
   float* ep = reinterpret_cast<float*>(&lds[0][0]);  // [0, 128): bias, [128, 256): s_x * s_w[c]
   float4 cb[MT == 1 ? 4 : 1], cs[MT == 1 ? 4 : 1];
   if constexpr (MT == 1) {
@@ -739,7 +772,7 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
       const int c0 = t_lo * 32;                      // first channel of the pass
       const int osz = o8 ? 1 : 2;
       const int valid = (cout_pad - c0) * osz;       // bytes of the pass row that exist
-      if (staged) {
+      if (staged && !(p == 0 && res_dma)) {   // (the first pass's residual tile is in the stage already)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int r = (lane >> 3) + 8 * j, c = lane & 7;

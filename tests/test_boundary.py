@@ -158,3 +158,18 @@ def test_compare_report_numbers_and_row_order_invariance(tmp_path, capsys):
                          "--dense-grid", "5x9x50", "--detail"]) == 0
     out = capsys.readouterr().out
     assert "[absdiff]: max:0.0" in out and "[absdiff = 0]: 100.000 %, 400" in out and "[cosine]: 100.000 %" in out
+
+
+def test_build_refuses_spills_in_kernels_with_counted_waits():
+    """The build reads the compiler's per-kernel resource remarks and fails when a kernel whose memory waits are
+    counted by hand uses scratch memory (a spill is a load those counts do not know about)."""
+    from lidar_ai_solution_amd import build as B
+    remark = "scn_conv_kernels.hpp:407:1: remark:     {} [-Rpass-analysis=kernel-resource-usage]"
+    def report(name, scratch):
+        return "\n".join([remark.format("Function Name: " + name), remark.format("VGPRs: 128"),
+                          remark.format(f"ScratchSize [bytes/lane]: {scratch}"), remark.format("Occupancy [waves/SIMD]: 4")])
+    lds = "_ZN3scn10k_conv_ldsILi0ELi4ELi4ELi8EEEvNS_8ConvArgsE"
+    out = "\n".join([report(lds, 0), report("_ZN3scn11k_conv_tileILi1ELi1ELi1EEEvNS_8ConvArgsE", 12),
+                     report(lds.replace("Li4ELi4", "Li2ELi4"), 256), "warning: something unrelated"])
+    assert B.kernels_with_scratch(out) == [(lds.replace("Li4ELi4", "Li2ELi4"), 256)]
+    assert B.kernels_with_scratch(report(lds, 0)) == []
