@@ -59,6 +59,8 @@ def _run(cmd, verbose):
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed: " + " ".join(cmd) + "\n" + out)
     if spilled:
+        if "-o" in cmd and os.path.exists(cmd[cmd.index("-o") + 1]):
+            os.remove(cmd[cmd.index("-o") + 1])   # (an incremental build must not pick the object up later)
         raise RuntimeError("kernels with hand-counted memory waits use scratch memory (register spills):\n" +
                            "\n".join(f"  {n}: {b} bytes per lane" for n, b in spilled))
     if verbose and out.strip():
