@@ -777,3 +777,49 @@ def test_launch_configuration_chosen_for_a_small_frame_serves_a_large_one(cp_mod
             g.replay()
             torch.cuda.synchronize()
             assert torch.equal(eng.output(0).torch().view(torch.int16), expect.view(torch.int16)), n_now
+
+
+def test_canonical_and_caller_order_inputs_give_the_same_bev(cp_models, centerpoint_input):
+    """Rows in canonical order (ascending linear voxel index) are indexed by rank, any other order through the
+    coordinate hash; the engine finds out which on the device.  The same voxels in both orders -- the reference's
+    frame as it ships (caller order) and sorted -- must give the same dense output bit for bit: direct forwards that
+    alternate between the two, then replays of one graph captured while the buffers held the canonical order, with the
+    buffers' contents exchanged between replays (more than 16 forwards, so the periodic second look happens)."""
+    feats, idx = centerpoint_input
+    _, g8 = cp_models
+    lin = (idx[:, 1].astype(np.int64) * GRID_ZYX[1] + idx[:, 2]) * GRID_ZYX[2] + idx[:, 3]
+    order = np.argsort(lin, kind="stable")
+    assert not np.array_equal(order, np.arange(order.size)), "the fixture is expected in caller order"
+    f_sorted, i_sorted = np.ascontiguousarray(feats[order]), np.ascontiguousarray(idx[order])
+    fresh = Engine.from_graph(g8, "int8")
+    _run_engine(fresh, feats, idx, GRID_ZYX)
+    want = fresh.output(0).torch().clone()
+    for aux in (False, True):
+        eng = Engine.from_graph(g8, "int8", with_auxiliary_stream=aux)
+        f, i = to_dev(f_sorted), to_dev(i_sorted)
+        eng.set_input(f, i, GRID_ZYX)
+        versions = [(torch.from_numpy(f_sorted).to(DEV), torch.from_numpy(i_sorted).to(DEV)),
+                    (torch.from_numpy(feats).to(DEV), torch.from_numpy(idx).to(DEV))]
+        note(f"direct forwards, orders alternating (auxiliary stream {aux})")
+        for k in range(20):
+            fv, iv = versions[(k // 2) % 2]
+            f.copy_(fv); i.copy_(iv)
+            eng.forward()
+            torch.cuda.synchronize()
+            assert torch.equal(eng.output(0).torch().view(torch.int16), want.view(torch.int16)), k
+        note("one graph captured on canonical rows, replayed on both orders")
+        f.copy_(versions[0][0]); i.copy_(versions[0][1])
+        eng.forward()
+        torch.cuda.synchronize()
+        st = torch.cuda.Stream()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=st):
+            eng.forward()
+        torch.cuda.synchronize()
+        for k in range(6):
+            fv, iv = versions[k % 2]
+            f.copy_(fv); i.copy_(iv)
+            assert np.isfinite(torch.randn(1 << 18, device=DEV).sum().item())
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(eng.output(0).torch().view(torch.int16), want.view(torch.int16)), k
