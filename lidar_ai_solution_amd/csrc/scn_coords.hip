@@ -105,13 +105,16 @@ __global__ __launch_bounds__(256) void k_hash_insert(uint64_t* slots, uint32_t m
                                                      uint32_t* n_eff_out, uint32_t* filter,
                                                      const uint32_t* skip_if_zero) {
   __shared__ uint32_t akeys[kAggSlots], avals[kAggSlots];
-  const uint32_t n = eff_n(n_dev, n_bound);
   const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
+  // (the flag first: a grid that only has to leave should not wait for the row count as well)
+  const bool skip = skip_if_zero && *skip_if_zero == 0;
+  if (skip && !(r == 0 && n_eff_out)) return;
+  const uint32_t n = eff_n(n_dev, n_bound);
   if (r == 0 && n_eff_out) {
     n_eff_out[0] = n;
     n_eff_out[1] = n;
   }
-  if (skip_if_zero && *skip_if_zero == 0) return;
+  if (skip) return;
   if (filter) agg_init(akeys, avals);
   uint32_t key;
   if (r < n && coord_key(coords[r], grid, &key)) {
@@ -122,36 +125,45 @@ __global__ __launch_bounds__(256) void k_hash_insert(uint64_t* slots, uint32_t m
 }
 
 // Rows in canonical order (strictly ascending linear index, every coordinate inside the grid): the first row of
-// every occupied 32-cell word ORs the bits of its run of rows (at most 32, consecutive) and writes the word and its
-// own row number with plain stores.  Any row that breaks the order raises *unsorted; what was written by then is
-// a subset of the true occupancy, which the hash insert that follows completes with its atomics.
+// every occupied 32-cell word writes the word's occupancy bits and its own row number.  The bits of a word's run of
+// rows (at most 32, consecutive) are combined inside the wavefront by a segmented suffix OR over lane shuffles; a run
+// that is whole inside one wavefront is written with a plain store, the two parts of one that crosses into the next
+// wavefront with an atomic OR each (the bitmap is cleared beforehand).  Any row that breaks the order raises
+// *unsorted; what was written by then is a subset of the true occupancy, which the hash insert that follows
+// completes with its atomics.
 __global__ __launch_bounds__(256) void k_index_sorted_rows(const int4* __restrict__ coords, uint32_t n_bound,
                                                            const uint32_t* n_dev, Int3 grid, uint32_t* bitmap,
                                                            uint32_t* first_row, uint32_t* unsorted) {
   const uint32_t n = eff_n(n_dev, n_bound);
   const uint32_t r = blockIdx.x * 256 + threadIdx.x;
-  if (r >= n) return;
-  uint32_t key;
-  if (!coord_key(coords[r], grid, &key)) {
-    *unsorted = 1u;
-    return;
+  const int lane = threadIdx.x & 63;
+  const bool have = r < n;
+  uint32_t key = 0;
+  const bool ok = have && coord_key(coords[r], grid, &key);
+  // the row before: the neighbouring lane's, or a load for the first lane of a wavefront
+  uint32_t kp = (uint32_t)__shfl_up((int)key, 1, 64);
+  bool okp = __shfl_up((int)ok, 1, 64) != 0;
+  if (lane == 0 && have && r > 0) okp = coord_key(coords[r - 1], grid, &kp);
+  if (have && (!ok || (r > 0 && (!okp || kp >= key)))) *unsorted = 1u;
+  const uint32_t word = ok ? key >> 5 : 0xFFFFFF00u + (uint32_t)lane;   // (rows without a cell never share a word)
+  const bool leader = ok && (r == 0 || !okp || (kp >> 5) != word);
+  uint32_t bits = ok ? 1u << (key & 31) : 0u;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const uint32_t ob = (uint32_t)__shfl_down((int)bits, d, 64);
+    const uint32_t ow = (uint32_t)__shfl_down((int)word, d, 64);
+    if (lane + d < 64 && ow == word) bits |= ob;   // equal words are contiguous, so the doubling covers the run
   }
-  if (r > 0) {
-    uint32_t kp;
-    if (!coord_key(coords[r - 1], grid, &kp) || kp >= key) {
-      *unsorted = 1u;
-      return;
-    }
-    if ((kp >> 5) == (key >> 5)) return;  // not the first row of its word
+  const bool reaches_end = (uint32_t)__shfl((int)word, 63, 64) == word;   // the run may go on in the next wavefront
+  if (leader) {
+    if (reaches_end)
+      atomicOr(&bitmap[word], bits);
+    else
+      bitmap[word] = bits;
+    first_row[word] = r;
+  } else if (lane == 0 && ok) {
+    atomicOr(&bitmap[word], bits);   // the part of a run that began in the wavefront before
   }
-  uint32_t bits = 1u << (key & 31);
-  for (uint32_t j = r + 1; j < n && j < r + 32; ++j) {
-    uint32_t kj;
-    if (!coord_key(coords[j], grid, &kj) || (kj >> 5) != (key >> 5)) break;
-    bits |= 1u << (kj & 31);
-  }
-  bitmap[key >> 5] = bits;
-  first_row[key >> 5] = r;
 }
 
 __global__ void k_hash_query(const uint64_t* __restrict__ slots, uint32_t mask, const int4* __restrict__ coords,
