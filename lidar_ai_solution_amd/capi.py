@@ -73,6 +73,7 @@ _SIGNATURES = {
     "scn_voxelizer_create": (vp, [C.POINTER(VoxelizationParam)]),
     "scn_voxelizer_destroy": (None, [vp]),
     "scn_voxelizer_forward": (C.c_int, [vp, vp, u32, C.c_int, vp]),
+    "scn_voxelizer_forward_points": (C.c_int, [vp, vp, C.c_int, u32, C.c_int, vp]),
     "scn_voxelizer_features": (vp, [vp]),
     "scn_voxelizer_indices": (vp, [vp]),
     "scn_voxelizer_num_voxels_dev": (vp, [vp]),

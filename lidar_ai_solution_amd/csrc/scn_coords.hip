@@ -913,8 +913,10 @@ struct VoxGeom {
   int max_voxels, max_pts;
 };
 
-// Pass 1 over the point stream: cell key per point + occupancy bit.
-__global__ __launch_bounds__(256) void k_vox_mark(const _Float16* __restrict__ pts, uint32_t n, VoxGeom g,
+// Pass 1 over the point stream (PT: fp16 points, or the fp32 points of CUDA-CenterPoint's preprocessing,
+// src/preprocess_kernels.cu:70-98): cell key per point + occupancy bit.
+template <typename PT>
+__global__ __launch_bounds__(256) void k_vox_mark(const PT* __restrict__ pts, uint32_t n, VoxGeom g,
                                                   uint32_t* pkey, uint32_t* bitmap) {
   const uint32_t p = blockIdx.x * 256 + threadIdx.x;
   if (p >= n) return;
@@ -960,7 +962,8 @@ __global__ __launch_bounds__(256) void k_vox_assign(const uint32_t* __restrict__
 }
 
 // Pass 3: per voxel mean of the kept points, summed in point-index order in fp32.
-__global__ __launch_bounds__(256) void k_vox_mean(const _Float16* __restrict__ pts, const uint32_t* n_vox_dev,
+template <typename PT>
+__global__ __launch_bounds__(256) void k_vox_mean(const PT* __restrict__ pts, const uint32_t* n_vox_dev,
                                                   int max_voxels, int max_pts, int nf,
                                                   const uint32_t* __restrict__ counts,
                                                   const uint32_t* __restrict__ mins, _Float16* feats) {
@@ -1073,9 +1076,17 @@ void scn_voxelizer_destroy(scn_voxelizer* v) {
 
 int scn_voxelizer_forward(scn_voxelizer* v, const void* points_fp16_dev, uint32_t num_points, int order,
                           void* stream_) {
+  return scn_voxelizer_forward_points(v, points_fp16_dev, SCN_DTYPE_FP16, num_points, order, stream_);
+}
+
+int scn_voxelizer_forward_points(scn_voxelizer* v, const void* points_fp16_dev, int points_dtype, uint32_t num_points,
+                                 int order, void* stream_) {
   SCN_REQUIRE(v, SCN_ERR_INVALID, "scn_voxelizer_forward: null voxelizer");
   SCN_REQUIRE(order == SCN_ORDER_XYZ || order == SCN_ORDER_ZYX, SCN_ERR_INVALID, "Invalid output_order: %d", order);
   SCN_REQUIRE(points_fp16_dev || num_points == 0, SCN_ERR_INVALID, "scn_voxelizer_forward: null points");
+  SCN_REQUIRE(points_dtype == SCN_DTYPE_FP16 || points_dtype == SCN_DTYPE_FP32, SCN_ERR_INVALID,
+              "scn_voxelizer_forward: points must be fp16 or fp32 (dtype %d)", points_dtype);
+  const bool p32 = points_dtype == SCN_DTYPE_FP32;
   hipStream_t stream = (hipStream_t)stream_;
   if (num_points > (uint32_t)v->p.max_points) {
     SCN_LOGW("voxelization: %u points exceed max_points %d, the frame is cropped", num_points, v->p.max_points);
@@ -1107,8 +1118,11 @@ int scn_voxelizer_forward(scn_voxelizer* v, const void* points_fp16_dev, uint32_
   if (rc) return rc;
   uint32_t* cnt = v->counters.as<uint32_t>();
   const uint32_t nblocks = (uint32_t)(v->words / kWordsPerBlock);
-  if (num_points)
-    hipLaunchKernelGGL(k_vox_mark, dim3(ceil_div(num_points, 256)), dim3(256), 0, stream,
+  if (num_points && p32)
+    hipLaunchKernelGGL(k_vox_mark<float>, dim3(ceil_div(num_points, 256)), dim3(256), 0, stream,
+                       (const float*)points_fp16_dev, num_points, g, v->pkey.as<uint32_t>(), v->bitmap.as<uint32_t>());
+  else if (num_points)
+    hipLaunchKernelGGL(k_vox_mark<_Float16>, dim3(ceil_div(num_points, 256)), dim3(256), 0, stream,
                        (const _Float16*)points_fp16_dev, num_points, g, v->pkey.as<uint32_t>(), v->bitmap.as<uint32_t>());
   hipLaunchKernelGGL(k_bitmap_blocksum, dim3(nblocks), dim3(256), 0, stream, v->bitmap.as<uint32_t>(),
                      v->blocksum.as<uint32_t>());
@@ -1122,9 +1136,14 @@ int scn_voxelizer_forward(scn_voxelizer* v, const void* points_fp16_dev, uint32_
                        num_points, v->bitmap.as<uint32_t>(), v->prefix.as<uint32_t>(), p.max_voxels,
                        p.max_points_per_voxel, v->counts.as<uint32_t>(), v->mins.as<uint32_t>());
     const uint32_t bound = (uint32_t)std::min<uint64_t>((uint64_t)p.max_voxels, num_points);
-    hipLaunchKernelGGL(k_vox_mean, dim3(ceil_div(bound * p.num_feature, 256)), dim3(256), 0, stream,
-                       (const _Float16*)points_fp16_dev, cnt, p.max_voxels, p.max_points_per_voxel, p.num_feature,
-                       v->counts.as<uint32_t>(), v->mins.as<uint32_t>(), (_Float16*)v->feats.p);
+    if (p32)
+      hipLaunchKernelGGL(k_vox_mean<float>, dim3(ceil_div(bound * p.num_feature, 256)), dim3(256), 0, stream,
+                         (const float*)points_fp16_dev, cnt, p.max_voxels, p.max_points_per_voxel, p.num_feature,
+                         v->counts.as<uint32_t>(), v->mins.as<uint32_t>(), (_Float16*)v->feats.p);
+    else
+      hipLaunchKernelGGL(k_vox_mean<_Float16>, dim3(ceil_div(bound * p.num_feature, 256)), dim3(256), 0, stream,
+                         (const _Float16*)points_fp16_dev, cnt, p.max_voxels, p.max_points_per_voxel, p.num_feature,
+                         v->counts.as<uint32_t>(), v->mins.as<uint32_t>(), (_Float16*)v->feats.p);
   }
   SCN_HIP(hipGetLastError());
   return SCN_OK;

@@ -303,7 +303,12 @@ class Voxelization:
         self.order = capi.ORDER_ZYX if order.lower() == "zyx" else capi.ORDER_XYZ
         n = int(points.shape[0] if num_points is None else num_points)
         self._keep = points
-        capi.check(capi.lib().scn_voxelizer_forward(self._h, C.c_void_p(points.data_ptr()), n, self.order, _stream_ptr(stream)))
+        import torch
+        if points.dtype not in (torch.float16, torch.float32):
+            raise ValueError("points must be a float16 or float32 device tensor")
+        dtype = capi.DTYPE_FP32 if points.dtype == torch.float32 else capi.DTYPE_FP16
+        capi.check(capi.lib().scn_voxelizer_forward_points(self._h, C.c_void_p(points.data_ptr()), dtype, n, self.order,
+                                                           _stream_ptr(stream)))
 
     def num_voxels(self, stream=None) -> int:
         return int(capi.lib().scn_voxelizer_num_voxels(self._h, _stream_ptr(stream)))

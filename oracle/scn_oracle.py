@@ -91,15 +91,19 @@ def set_num_threads(n: int) -> None:
 # ------------------------------------------------------------------------------- voxelization
 def voxelize(points_f16: np.ndarray, min_range, max_range, voxel_size, grid_xyz, max_voxels=160000,
              max_points=10, order="zyx"):
-    """Returns (features [nv, F] fp16, indices [nv, 4] int32, points_per_voxel [nv] int32)."""
-    pts = np.ascontiguousarray(points_f16, dtype=np.float16)
+    """Returns (features [nv, F] fp16, indices [nv, 4] int32, points_per_voxel [nv] int32).  Points are taken as
+    fp16 unless the array is float32 (the raw sweep of CUDA-CenterPoint's preprocessing)."""
+    f32 = np.asarray(points_f16).dtype == np.float32
+    pts = np.ascontiguousarray(points_f16, dtype=np.float32 if f32 else np.float16)
     n, nf = pts.shape
     feats = np.zeros((max_voxels, nf), np.float16)
     idx = np.zeros((max_voxels, 4), np.int32)
     cnt = np.zeros((max_voxels,), np.int32)
-    nv = lib().scn_ref_voxelize(_p(pts.view(np.uint16)), C.c_int(n), C.c_int(nf), _f3(min_range), _f3(max_range),
-                                _f3(voxel_size), _i3(grid_xyz), C.c_int(max_voxels), C.c_int(max_points),
-                                C.c_int(2 if order == "zyx" else 1), _p(feats.view(np.uint16)), _p(idx), _p(cnt))
+    fn = lib().scn_ref_voxelize_f32 if f32 else lib().scn_ref_voxelize
+    fn.restype = C.c_int
+    nv = fn(_p(pts if f32 else pts.view(np.uint16)), C.c_int(n), C.c_int(nf), _f3(min_range), _f3(max_range),
+            _f3(voxel_size), _i3(grid_xyz), C.c_int(max_voxels), C.c_int(max_points),
+            C.c_int(2 if order == "zyx" else 1), _p(feats.view(np.uint16)), _p(idx), _p(cnt))
     return feats[:nv].copy(), idx[:nv].copy(), cnt[:nv].copy()
 
 

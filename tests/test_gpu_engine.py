@@ -823,3 +823,34 @@ def test_canonical_and_caller_order_inputs_give_the_same_bev(cp_models, centerpo
             g.replay()
             torch.cuda.synchronize()
             assert torch.equal(eng.output(0).torch().view(torch.int16), want.view(torch.int16)), k
+
+
+def test_cpp_centerpoint_preprocessing_and_legacy_engine_on_a_raw_fp32_sweep(cp_models, nuscenes_frame, tmp_path):
+    """The lidar half of CUDA-CenterPoint's CenterPoint::doinfer (src/centerpoint.cpp:136-150) as a C++ program:
+    PreProcessCuda::generateVoxels(const float*) / getOutput (include/legacy/preprocess.h) feed the older single-call
+    engine interface.  Voxels must equal the oracle's for the fp32 points bit for bit, the BEV tensor the Python
+    engine's on those voxels."""
+    import subprocess
+    from lidar_ai_solution_amd import tensor
+    exe = _example("centerpoint_pre")
+    rng = np.random.default_rng(4)
+    pts = nuscenes_frame[:200000].astype(np.float32)
+    pts[:, :3] += rng.uniform(-0.03, 0.03, (pts.shape[0], 3)).astype(np.float32)
+    pts.tofile(str(tmp_path / "sweep.bin"))
+    model = str(tmp_path / "cp.int8.scn.onnx")
+    onnx_dialect.save(cp_models[1], model)
+    prefix = str(tmp_path / "cp")
+    note("centerpoint_pre on a 200,000-point fp32 sweep")
+    r = subprocess.run([exe, model, str(tmp_path / "sweep.bin"), "int8", prefix], stdout=subprocess.PIPE,
+                       stderr=subprocess.STDOUT, text=True, timeout=180)
+    print(r.stdout)
+    assert r.returncode == 0, r.stdout
+    rf, ri, _ = O.voxelize(pts, synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, order="zyx")
+    gf, gi = tensor.load(prefix + ".features.tensor"), tensor.load(prefix + ".indices.tensor")
+    assert np.array_equal(gi, ri) and np.array_equal(gf.view(np.uint16), rf.view(np.uint16))
+    assert f"sparse_shape: {GRID_ZYX[0]} x {GRID_ZYX[1]} x {GRID_ZYX[2]}" in r.stdout
+    eng = Engine.from_onnx(model, "int8")
+    _run_engine(eng, rf, ri, GRID_ZYX)
+    got = tensor.load(prefix + ".bev.tensor")
+    assert got.shape == (1, 256, 180, 180)
+    assert np.array_equal(got.view(np.uint16), eng.output(0).torch().cpu().numpy().view(np.uint16))

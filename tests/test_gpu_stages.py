@@ -663,7 +663,10 @@ def _run_voxelizer(h, pts, order, max_voxels):
     L = capi.lib()
     code = capi.ORDER_ZYX if order == "zyx" else capi.ORDER_XYZ
     d = to_dev(pts)
-    capi.check(L.scn_voxelizer_forward(h, ptr(d), pts.shape[0], code, stream()))
+    if pts.dtype == np.float32:
+        capi.check(L.scn_voxelizer_forward_points(h, ptr(d), capi.DTYPE_FP32, pts.shape[0], code, stream()))
+    else:
+        capi.check(L.scn_voxelizer_forward(h, ptr(d), pts.shape[0], code, stream()))
     nv = L.scn_voxelizer_num_voxels(h, stream())
     f = copy_from_ptr(L.scn_voxelizer_features(h), (nv, 5), np.float16).cpu().numpy()
     i = copy_from_ptr(L.scn_voxelizer_indices(h), (nv, 4), np.int32).cpu().numpy()
@@ -692,6 +695,35 @@ def test_voxelization_real_frame_bit_exact(order, nuscenes_frame):
         assert np.array_equal(i2, ri2) and np.array_equal(c2, rc2) and np.array_equal(f2.view(np.uint16), rf2.view(np.uint16))
         f0, i0, _ = _run_voxelizer(h, pts2[:0], order, 160000)
         assert f0.shape[0] == 0
+    finally:
+        L.scn_voxelizer_destroy(h)
+
+
+@pytest.mark.parametrize("order", ["zyx", "xyz"])
+def test_voxelization_of_fp32_points_bit_exact(order, nuscenes_frame):
+    """The raw fp32 sweep, as CUDA-CenterPoint's preprocessing takes it (PreProcessCuda::generateVoxels(const float*),
+    src/preprocess.cpp:82, src/preprocess_kernels.cu:70-154): coordinates that no fp16 value represents, so that the
+    range test, the cell index and the fp32 sums really run on the fp32 values."""
+    rng = np.random.default_rng(9)
+    pts = nuscenes_frame[:150000].astype(np.float32)
+    pts[:, :3] += rng.uniform(-0.03, 0.03, (pts.shape[0], 3)).astype(np.float32)
+    pts[:, 3] *= np.float32(1.0009765)
+    assert not np.array_equal(pts, pts.astype(np.float16).astype(np.float32))
+    note(f"voxelization of {pts.shape[0]} fp32 points, order {order}")
+    L = capi.lib()
+    h = _voxelizer()
+    try:
+        f, i, c = _run_voxelizer(h, pts, order, 160000)
+        rf, ri, rc = O.voxelize(pts, synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, order=order)
+        assert np.array_equal(i, ri) and np.array_equal(c, rc)
+        assert np.array_equal(f.view(np.uint16), rf.view(np.uint16))
+        # ... and differs from what the fp16-rounded points give (another set of cells)
+        r16 = O.voxelize(pts.astype(np.float16), synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, order=order)
+        assert r16[1].shape != ri.shape or not np.array_equal(r16[1], ri)
+        note("an fp16 frame on the same object afterwards")
+        f2, i2, c2 = _run_voxelizer(h, nuscenes_frame[:50000], order, 160000)
+        rf2, ri2, rc2 = O.voxelize(nuscenes_frame[:50000], synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, order=order)
+        assert np.array_equal(i2, ri2) and np.array_equal(c2, rc2) and np.array_equal(f2.view(np.uint16), rf2.view(np.uint16))
     finally:
         L.scn_voxelizer_destroy(h)
 

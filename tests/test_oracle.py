@@ -117,6 +117,21 @@ def test_voxelize_against_brute_force(order, nuscenes_frame):
     assert n.max() > 10  # the crowded-voxel rule is exercised
 
 
+@pytest.mark.parametrize("order", ["zyx", "xyz"])
+def test_voxelize_fp32_points_against_brute_force(order, nuscenes_frame):
+    """fp32 points (CUDA-CenterPoint's preprocessing, src/preprocess_kernels.cu:70-154) that no fp16 value represents."""
+    rng = np.random.default_rng(9)
+    pts = nuscenes_frame[:40000].astype(np.float32)
+    pts[:, :3] += rng.uniform(-0.03, 0.03, (pts.shape[0], 3)).astype(np.float32)
+    assert not np.array_equal(pts, pts.astype(np.float16).astype(np.float32))
+    f, c, n = O.voxelize(pts, synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, order=order)
+    bf, bc, bn, _ = _brute_voxelize(pts, order)
+    assert np.array_equal(c, bc)
+    assert np.array_equal(n, bn)
+    assert np.array_equal(f.view(np.uint16), bf.view(np.uint16))
+    assert n.max() > 10
+
+
 def test_voxelize_known_answer_full_frame(nuscenes_frame):
     ka = KNOWN["nuscenes_frame"]
     assert nuscenes_frame.shape[0] == ka["points"]
