@@ -1110,11 +1110,11 @@ int scn_voxelizer_forward_points(scn_voxelizer* v, const void* points_fp16_dev, 
   g.max_voxels = p.max_voxels;
   g.max_pts = p.max_points_per_voxel;
   v->last_order = order;
-  int rc = fill_u32(v->bitmap.p, 0u, v->words, stream);
-  if (rc) return rc;
-  rc = fill_u32(v->mins.p, 0xFFFFFFFFu, (size_t)p.max_voxels * p.max_points_per_voxel, stream);
-  if (rc) return rc;
-  rc = fill_u32(v->counts.p, 0u, (size_t)p.max_voxels, stream);
+  // one launch clears the cell bitmap, the per-voxel point slots and the per-voxel counts
+  const FillJob clears[3] = {{v->bitmap.p, v->words, 0u},
+                             {v->mins.p, (size_t)p.max_voxels * p.max_points_per_voxel, 0xFFFFFFFFu},
+                             {v->counts.p, (size_t)p.max_voxels, 0u}};
+  int rc = fill_multi(clears, 3, nullptr, nullptr, 0, stream);
   if (rc) return rc;
   uint32_t* cnt = v->counters.as<uint32_t>();
   const uint32_t nblocks = (uint32_t)(v->words / kWordsPerBlock);
