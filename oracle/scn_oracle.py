@@ -23,6 +23,12 @@ Precision rules stated by this build (the closed engine's are not recoverable):
   * SparseInverseConvolution (parity unpinned: no reference vector exists): the transposed convolution
     on the named strided rulebook, out[i] += W[k] x[o] for each of its pairs (i, o, k), kernel not
     flipped; pinned against torch's conv_transpose3d under that rule.
+  * dense output forms (engine.hpp:26,114-123): NCHW32 / NHWzC are defined by their names over the
+    [1, C * Z, H, W] view the exporters' tails build; an int8 dense output (the node carries
+    input_dynamic_range) holds the fake-quantised fp32 value of every element at that range, and a tensor
+    no convolution or Add reads is stored int8 with the dense node's range.  The closed engine's byte layout
+    is not observable; the definitions are pinned element by element with explicit index arithmetic and an
+    independent dense walk (tests/test_oracle_graph.py).
 """
 from __future__ import annotations
 

@@ -124,6 +124,10 @@ def _pushed_ranges(graph, kinds):
             for slot in (0, 1):
                 rng.setdefault(n.inputs[slot], F32(n.attrs[f"input{slot}_dynamic_range"]))
     through_relus()
+    for n in graph.nodes:   # an int8 dense output quantises with its own range a tensor nobody else fixed
+        if n.op_type == "ScatterDense" and float(n.attrs.get("input_dynamic_range", 0.0) or 0.0) > 0:
+            rng.setdefault(n.inputs[0], F32(n.attrs["input_dynamic_range"]))
+    through_relus()
     return rng
 
 
@@ -144,6 +148,7 @@ def dense_walk(graph, feats, idx, grid, precision, record=None, rebase=None, add
     m0[idx[:, 1], idx[:, 2], idx[:, 3]] = 1.0
     T = {graph.inputs[0]: Dense(x0, m0)}
     strided_in = {}   # rulebook key -> (mask, grid) of the strided convolution's input
+    fixed_form = set()
 
     def value(t: Dense):
         """fp32 value of every stored element."""
@@ -220,8 +225,12 @@ def dense_walk(graph, feats, idx, grid, precision, record=None, rebase=None, add
             t = T[n.inputs[0]]
             T[name] = Dense(np.maximum(t.val, 0.0), t.mask, t.rng)
         elif n.op_type == "ScatterDense":
-            t = T[n.inputs[0]]
-            T[name] = value(t).astype(np.float16)[None]            # [1, C, D0, D1, D2], zero outside the mask
+            T[name], fixed = dense_tail(T[n.inputs[0]], n, precision)   # [1, C, D0, D1, D2], zero outside the mask
+            if fixed:
+                fixed_form.add(name)
+        elif n.op_type in ("Reshape", "Transpose") and n.inputs[0] in fixed_form:
+            T[name] = T[n.inputs[0]]          # a vectorised layout already is the final tensor
+            fixed_form.add(name)
         elif n.op_type == "Reshape":
             T[name] = np.ascontiguousarray(T[n.inputs[0]]).reshape([int(v) for v in a["dims"]])
         elif n.op_type == "Transpose":
@@ -453,3 +462,134 @@ def test_one_range_per_tensor_against_per_consumer_fake_quant():
         worst = max(worst, diff / step)
     print(f"one range per tensor vs per-consumer fake-quant: worst difference {worst:.3f} quantisation steps")
     assert worst <= 0.5 + 1e-6
+
+
+# ------------------------------------------------------------------------------------------ dense output forms
+# push_dense's vectorised layouts and int8 output (engine.hpp:26,114-123; src/onnx-parser.cpp:196-203).  The
+# definitions are closed forms over the [1, C * Z, H, W] tensor the exporters' tails build (channel c * Z + z:
+# tool/centerpoint-export/exptool.py:159-183 for zyx, CUDA-BEVFusion/qat/lean/exptool.py:285-293 for xyz, whose
+# dense tensor is [1, C, X, Y, Z] and whose H, W are X, Y).  They are written here element by element with
+# explicit index arithmetic; nothing below calls numpy's transpose or reshape on the data.
+def _view_axes(fmt, d0, d1, d2):
+    """(Z, H, W) and a function (z, h, w) -> (i0, i1, i2) of the [1, C, D0, D1, D2] dense tensor."""
+    if fmt == "zyx":
+        return (d0, d1, d2), (lambda z, h, w: (z, h, w))
+    return (d2, d0, d1), (lambda z, h, w: (h, w, z))
+
+
+def layout_by_index_arithmetic(dense, fmt, layout, swap_z_and_c=False):
+    _, C, d0, d1, d2 = dense.shape
+    (Z, H, W), at = _view_axes(fmt, d0, d1, d2)
+    if layout == "NCHW32":
+        groups = (C * Z + 31) // 32
+        flat = np.zeros(groups * H * W * 32, dense.dtype)
+        shape = (1, groups, H, W, 32)
+    elif layout == "NHWzC":
+        flat = np.zeros(H * W * Z * C, dense.dtype)
+        shape = (1, H, W, Z, C)
+    else:
+        flat = np.zeros(C * Z * H * W, dense.dtype)
+        shape = (1, C * Z, H, W)
+    for c in range(C):
+        for z in range(Z):
+            cz = c * Z + z
+            for h in range(H):
+                for w in range(W):
+                    v = dense[(0, c) + at(z, h, w)]
+                    if layout == "NCHW32":
+                        flat[(((cz // 32) * H + h) * W + w) * 32 + cz % 32] = v
+                    elif layout == "NHWzC":
+                        flat[(((h * W + w) * C + c) * Z + z) if swap_z_and_c else (((h * W + w) * Z + z) * C + c)] = v
+                    else:
+                        flat[(cz * H + h) * W + w] = v
+    return flat.reshape(shape)
+
+
+@pytest.mark.parametrize("fmt", ["zyx", "xyz"])
+def test_dense_to_layout_by_explicit_index_arithmetic(fmt):
+    """Every element distinct, C * Z = 48 so that NCHW32 pads its second group with zeros."""
+    C, Z, H, W = 24, 2, 5, 7
+    dims = (Z, H, W) if fmt == "zyx" else (H, W, Z)
+    dense = (np.arange(C * Z * H * W, dtype=np.int32) + 1).reshape(1, C, *dims).astype(np.float32).astype(np.float16)
+    assert len(np.unique(dense)) == dense.size   # 1 .. 1680 are exact in fp16
+    for layout in ("NCHW32", "NHWzC"):
+        want = layout_by_index_arithmetic(dense, fmt, layout)
+        got = O.dense_to_layout(dense, fmt, layout)
+        assert got.shape == want.shape and np.array_equal(got, want), (fmt, layout)
+    pad = O.dense_to_layout(dense, fmt, "NCHW32")
+    assert pad.shape == (1, 2, H, W, 32) and np.count_nonzero(pad[0, 1, :, :, 16:]) == 0 and np.count_nonzero(pad) == dense.size
+    # sensitivity: a definition with z and C swapped in NHWzC, or the other format's axis convention, is a different tensor
+    assert not np.array_equal(layout_by_index_arithmetic(dense, fmt, "NHWzC", swap_z_and_c=True).ravel(),
+                              O.dense_to_layout(dense, fmt, "NHWzC").ravel())
+    other = "xyz" if fmt == "zyx" else "zyx"
+    wrong_axes = np.ascontiguousarray(dense.reshape(1, C, *((H, W, Z) if fmt == "zyx" else (Z, H, W))))
+    assert not np.array_equal(O.dense_to_layout(wrong_axes, other, "NCHW32").ravel(), pad.ravel())
+    # the plain NCHW tail of the exporters, by the same arithmetic, against their own numpy calls
+    tail = dense.reshape(1, C * Z, H, W) if fmt == "zyx" else np.transpose(dense, (0, 1, 4, 2, 3)).reshape(1, C * Z, H, W)
+    assert np.array_equal(layout_by_index_arithmetic(dense, fmt, "NCHW"), tail)
+
+
+def dense_tail(t: Dense, node, precision):
+    """Independent restatement of a ScatterDense node: the fp32 value of every stored element as fp16, or, for an
+    int8 output (the node carries input_dynamic_range and the engine runs int8), that value fake-quantised with
+    the node's own range; zero outside the active set either way; then the layout by index arithmetic.
+    Returns (tensor, True when it is in a vectorised layout that the Transpose / Reshape tail leaves alone)."""
+    a = node.attrs
+    val = t.val.astype(F32) if t.rng is None else t.val.astype(F32) * (F32(t.rng) / F32(127.0))
+    out_rng = float(a.get("input_dynamic_range", 0.0) or 0.0)
+    if out_rng > 0 and precision == "int8":
+        dense = (_quant(val, out_rng) * t.mask[None]).astype(np.int8)[None]
+    else:
+        dense = val.astype(np.float16)[None]
+    layout = a.get("output_layout", "") or "NCHW"
+    if layout == "NCHW":
+        return dense, False
+    return layout_by_index_arithmetic(dense, a.get("format", "zyx"), layout), True
+
+
+@pytest.mark.parametrize("kind,data_fn,layout,int8_out,plan", [
+    ("centerpoint", _cp, "NCHW32", True, "all-int8"), ("centerpoint", _cp, "NCHW", True, "all-int8"),
+    ("bevfusion", _bev, "NHWzC", False, "all-int8"), ("bevfusion", _bev, "NCHW32", True, "all-int8"),
+    ("bevfusion", _bev, "NHWzC", True, "all-int8"), ("centerpoint", _cp, "NCHW32", False, "all-int8"),
+    ("bevfusion", _bev, "NCHW", True, "bevfusion")])   # (last: the tensor in front of the dense node is stored fp16)
+def test_dense_output_forms_of_the_graph_walk_against_dense_walk(kind, data_fn, layout, int8_out, plan):
+    """run_graph's ScatterDense branch for int8 output and the vectorised layouts, and the rule that the tensor
+    feeding an int8 dense node is stored int8 with that node's range when no other consumer fixes one, against
+    the dense walk (ranges pushed from consumers, dense_tail, layouts by index arithmetic)."""
+    data = data_fn()
+    feats, idx, grid = data
+    g = _graph(kind, 21, plan, data)
+    sd = [n for n in g.nodes if n.op_type == "ScatterDense"][0]
+    sd.attrs["output_layout"] = layout
+    last_conv = [n for n in g.nodes if n.outputs[0] == sd.inputs[0]][0]
+    if int8_out:
+        # a range that clips some values, so that the clamp and the choice of range both show
+        rec = {}
+        dense_walk(g, feats, idx, grid, "int8", rec)
+        t = rec[last_conv.name]
+        sd.attrs["input_dynamic_range"] = float(0.6 * np.abs(t.val[:, t.mask > 0]).max())
+    rec_o, rec_d = {}, {}
+    got = O.run_graph(g, feats, idx, grid, "int8", rec_o)[g.outputs[0]]
+    rebase = None
+    if plan != "all-int8":
+        # conv_input computes in fp16 (summation order): continue the dense walk from the oracle's result of it
+        n0 = g.nodes[0]
+        v, m = to_dense(T_of(rec_o, None, g, n0))
+        rebase = {n0.outputs[0]: Dense(v, m, None if rec_o[n0.name]["range"] is None else F32(rec_o[n0.name]["range"]))}
+    want = dense_walk(g, feats, idx, grid, "int8", rec_d, rebase=rebase)[g.outputs[0]]
+    if int8_out and plan == "all-int8":
+        assert F32(rec_o[last_conv.name]["range"]) == F32(rec_d[last_conv.name].rng) == F32(sd.attrs["input_dynamic_range"])
+    else:   # stored fp16: by the plan, or because nothing downstream quantises
+        assert rec_o[last_conv.name]["range"] is None and rec_d[last_conv.name].rng is None
+    assert got.dtype == want.dtype == (np.int8 if int8_out else np.float16)
+    c3, z = CHANNELS[3], 2
+    expect = {"NCHW32": (1, (c3 * z + 31) // 32, 8, 8, 32), "NHWzC": (1, 8, 8, z, c3), "NCHW": (1, c3 * z, 8, 8)}[layout]
+    assert got.shape == want.shape == expect, (got.shape, want.shape)
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    assert np.count_nonzero(got) > 50
+    if int8_out:
+        assert np.abs(got).max() == 127 and np.mean(np.abs(got[got != 0]) == 127) < 0.5   # the range clips, not everywhere
+        # sensitivity: quantising the dense output from the stored fp16-rounded value instead of from the int8 code's
+        # value, or with the conv's weight range, is caught because the range differs from every other in the graph
+        assert all(F32(n.attrs.get("input_dynamic_range", -1)) != F32(sd.attrs["input_dynamic_range"])
+                   for n in g.nodes if n is not sd)
