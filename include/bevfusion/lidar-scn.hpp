@@ -53,6 +53,7 @@ class SCNImplement : public SCN {
   }
   const nvtype::half* forward(const nvtype::half* points, unsigned int num_points, void* stream) override {
     voxelization_->forward(points, (int)num_points, stream, param_.order);
+    if (!voxelization_->last_forward_ok()) return nullptr;   // (logged there; the backbone must not run on stale voxels)
     auto* in = native_scn_->input(0);
     const int64_t cap = voxelization_->max_voxels();
     in->features().reference(const_cast<void*>(voxelization_->features()), {cap, (int64_t)voxelization_->voxel_dim()},

@@ -15,6 +15,7 @@
 
 #include "../common/dtype.hpp"
 #include "../scn_c_api.h"
+#include "../spconv/engine.hpp"
 
 namespace bevfusion {
 namespace lidar {
@@ -59,6 +60,9 @@ class Voxelization {
   // not in the reference: what a caller needs to hand the result on without a host round trip
   virtual const unsigned int* num_voxels_device() = 0;
   virtual unsigned int max_voxels() = 0;
+  // false after a forward() that failed (invalid order, null points, launch error): the buffers then still hold the
+  // previous frame and num_voxels() reports 0.  (forward() itself returns nothing, as in the reference.)
+  virtual bool last_forward_ok() { return true; }
 };
 
 namespace detail {
@@ -84,9 +88,12 @@ class VoxelizationImplement : public Voxelization {
   void forward(const nvtype::half* points, int num_points, void* stream, CoordinateOrder output_order) override {
     order_ = output_order;
     stream_ = stream;
-    (void)scn_voxelizer_forward(v_, points, (uint32_t)(num_points < 0 ? 0 : num_points), (int)output_order, stream);
+    rc_ = scn_voxelizer_forward(v_, points, (uint32_t)(num_points < 0 ? 0 : num_points), (int)output_order, stream);
+    if (rc_ != SCN_OK)
+      spconv::logger_output(__FILE__, __LINE__, spconv::LoggerLevel::Error, "voxelization failed (%d): %s", rc_, scn_last_error());
   }
-  unsigned int num_voxels() override { return scn_voxelizer_num_voxels(v_, stream_); }
+  bool last_forward_ok() override { return rc_ == SCN_OK; }
+  unsigned int num_voxels() override { return rc_ == SCN_OK ? scn_voxelizer_num_voxels(v_, stream_) : 0u; }
   unsigned int voxel_dim() override { return (unsigned int)param_.num_feature; }
   unsigned int indices_dim() override { return 4; }
   std::vector<int> grid_size() override {
@@ -105,6 +112,7 @@ class VoxelizationImplement : public Voxelization {
   scn_voxelizer* v_ = nullptr;
   CoordinateOrder order_ = CoordinateOrder::XYZ;
   void* stream_ = nullptr;
+  int rc_ = SCN_OK;
 };
 }  // namespace detail
 

@@ -76,6 +76,7 @@ class PreProcessCuda {
     stream_ = stream;
     const int rc = scn_voxelizer_forward_points(vox_, points, SCN_DTYPE_FP32, (uint32_t)points_size, SCN_ORDER_ZYX, stream);
     if (rc != 0) fprintf(stderr, "PreProcessCuda::generateVoxels: %s\n", scn_last_error());
+    last_rc_ = rc;
     return rc;
   }
 
@@ -83,7 +84,7 @@ class PreProcessCuda {
   // the sparse shape {Z + 1, Y, X}, and n (this waits for the stream of the last generateVoxels)
   unsigned int getOutput(half** d_voxel_features, unsigned int** d_voxel_indices, std::vector<int>& sparse_shape) {
     sparse_shape.clear();
-    if (!vox_) return 0;
+    if (!vox_ || last_rc_ != 0) return 0;   // (after a failed call the buffers still hold the previous frame)
     *d_voxel_features = (half*)scn_voxelizer_features(vox_);
     *d_voxel_indices = (unsigned int*)scn_voxelizer_indices(vox_);
     int g[3];
@@ -99,6 +100,7 @@ class PreProcessCuda {
   Params params_;
   scn_voxelizer* vox_ = nullptr;
   hipStream_t stream_ = nullptr;
+  int last_rc_ = 0;
 };
 
 #endif  // SCN_LEGACY_PREPROCESS_H

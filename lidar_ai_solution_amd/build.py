@@ -67,12 +67,25 @@ def _run(cmd, verbose):
         print(out)
 
 
-def _stale(obj: str, src: str) -> bool:
-    """True when obj is older than its source or than any header of csrc/ and include/."""
-    if not os.path.exists(obj):
+def _stamp(cmd) -> str:
+    """What an object file was compiled with: the command line (flags, include paths) and the list of kernels whose
+    scratch use fails the build.  Kept next to the object; an object whose stamp differs is compiled again, so that
+    the scratch check has run with the current rules on everything that is linked."""
+    import hashlib
+    return hashlib.sha256(("\0".join(cmd) + "\0" + ",".join(NO_SCRATCH_KERNELS)).encode()).hexdigest()
+
+
+def _stale(obj: str, src: str, cmd) -> bool:
+    """True when obj is older than its source or than any header of csrc/ and include/ (all levels), or was
+    compiled with another command line."""
+    if not os.path.exists(obj) or not os.path.exists(obj + ".stamp"):
         return True
+    with open(obj + ".stamp") as f:
+        if f.read().strip() != _stamp(cmd):
+            return True
     t = os.path.getmtime(obj)
-    deps = [src] + glob.glob(os.path.join(HERE, "csrc", "*.hpp")) + glob.glob(os.path.join(ROOT, "include", "*.h"))
+    deps = [src] + glob.glob(os.path.join(HERE, "csrc", "*.hpp")) + \
+        [p for p in glob.glob(os.path.join(ROOT, "include", "**", "*"), recursive=True) if os.path.isfile(p)]
     return any(os.path.getmtime(d) > t for d in deps)
 
 
@@ -91,12 +104,22 @@ def build(verbose: bool = False, jobs: int = 0, incremental: bool = False) -> st
     for src in sources():
         obj = os.path.join(obj_dir, os.path.basename(src) + ".o")
         objs.append(obj)
-        if incremental and not _stale(obj, src):
-            continue
         remarks = [RESOURCE_REMARKS] if os.path.basename(src).startswith("scn_conv_") else []
-        cmds.append(["hipcc", *compile_flags, *remarks, "-I" + os.path.join(ROOT, "include"), "-c", src, "-o", obj])
+        cmd = ["hipcc", *compile_flags, *remarks, "-I" + os.path.join(ROOT, "include"), "-c", src, "-o", obj]
+        if incremental and not _stale(obj, src, cmd):
+            continue
+        cmds.append(cmd)
+
+    def compile_one(cmd):
+        obj = cmd[cmd.index("-o") + 1]
+        if os.path.exists(obj + ".stamp"):
+            os.remove(obj + ".stamp")
+        _run(cmd, verbose)
+        with open(obj + ".stamp", "w") as f:
+            f.write(_stamp(cmd))
+
     with ThreadPoolExecutor(max_workers=jobs_) as pool:
-        list(pool.map(lambda c: _run(c, verbose), cmds))
+        list(pool.map(compile_one, cmds))
     _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-fvisibility=hidden", "-no-hip-rt", *objs, "-o", LIB_PATH],
          verbose)
     return LIB_PATH

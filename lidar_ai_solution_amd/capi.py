@@ -63,6 +63,8 @@ _SIGNATURES = {
     "scn_device_bytes_in_use": (C.c_size_t, []),
     "scn_set_log_level": (None, [C.c_int]),
     "scn_get_log_level": (C.c_int, []),
+    "scn_set_debug_sync": (None, [C.c_int]),
+    "scn_get_debug_sync": (C.c_int, []),
     "scn_set_log_callback": (None, [LOG_CALLBACK, vp]),
     "scn_log": (None, [C.c_char_p, C.c_int, C.c_int, C.c_char_p]),
     "scn_memset_async": (C.c_int, [vp, C.c_ubyte, C.c_size_t, vp]),
@@ -124,6 +126,7 @@ _SIGNATURES = {
     "scn_builder_build": (vp, [vp, C.c_int, C.c_uint, vp]),
     "scn_engine_create_from_onnx": (vp, [C.c_char_p, C.c_int, C.c_uint, C.c_uint, vp]),
     "scn_engine_create_from_onnx_ex": (vp, [C.c_char_p, C.c_int, C.c_uint, C.c_uint, vp, vp]),
+    "scn_engine_create_from_onnx_memory": (vp, [vp, C.c_size_t, C.c_int, C.c_uint, C.c_uint, vp, vp]),
     "scn_engine_collect_amax": (C.c_int, [vp, vp, vp, C.c_int]),
     "scn_engine_destroy": (None, [vp]),
     "scn_engine_num_input": (C.c_int, [vp]),

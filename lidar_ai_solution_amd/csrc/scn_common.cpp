@@ -2,6 +2,7 @@
 #include "scn_common.hpp"
 
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 
@@ -11,6 +12,25 @@ static int g_level = kWarn;
 static scn_log_callback g_cb = nullptr;
 static void* g_cb_user = nullptr;
 static thread_local std::string g_last_error;
+static int g_debug_sync = -1;   // -1: not decided yet (SCN_DEBUG_SYNC in the environment decides on first use)
+
+bool debug_sync_enabled() {
+  if (g_debug_sync < 0) {
+    const char* e = getenv("SCN_DEBUG_SYNC");
+    g_debug_sync = (e && *e && strcmp(e, "0") != 0) ? 1 : 0;
+  }
+  return g_debug_sync != 0;
+}
+
+int debug_sync_check(hipStream_t stream, const char* what) {
+  hipError_t err = hipStreamSynchronize(stream);
+  if (err == hipSuccess) err = hipGetLastError();
+  if (err != hipSuccess) {
+    set_error("debug sync: %s failed: %s", what, hipGetErrorString(err));
+    return SCN_ERR_HIP;
+  }
+  return SCN_OK;
+}
 
 static const char* level_name(int level) {
   switch (level) {
@@ -115,6 +135,8 @@ size_t scn_device_bytes_in_use(void) { return scn::device_bytes_counter().load()
 const char* scn_last_error(void) { return scn::g_last_error.c_str(); }
 void scn_set_log_level(int level) { scn::g_level = level; }
 int scn_get_log_level(void) { return scn::g_level; }
+void scn_set_debug_sync(int enabled) { scn::g_debug_sync = enabled ? 1 : 0; }
+int scn_get_debug_sync(void) { return scn::debug_sync_enabled() ? 1 : 0; }
 void scn_set_log_callback(scn_log_callback cb, void* user) {
   scn::g_cb = cb;
   scn::g_cb_user = user;

@@ -19,6 +19,12 @@ enum LogLevel : int { kVerb = 0, kWarn = 1, kError = 2, kQuiet = 99 };
 void log_message(const char* file, int line, int level, const char* fmt, ...) __attribute__((format(printf, 4, 5)));
 void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 
+// Debug mode (SCN_DEBUG_SYNC=1 in the environment, or scn_set_debug_sync): every step of a forward and every stage-level
+// entry point waits for its kernels and reports an asynchronous failure with the step's name, instead of letting it
+// surface at some later call.  Not for captured graphs (it synchronises) and not for timing.
+bool debug_sync_enabled();
+int debug_sync_check(hipStream_t stream, const char* what);
+
 #define SCN_LOGV(...) ::scn::log_message(__FILE__, __LINE__, ::scn::kVerb, __VA_ARGS__)
 #define SCN_LOGW(...) ::scn::log_message(__FILE__, __LINE__, ::scn::kWarn, __VA_ARGS__)
 #define SCN_LOGE(...) ::scn::log_message(__FILE__, __LINE__, ::scn::kError, __VA_ARGS__)

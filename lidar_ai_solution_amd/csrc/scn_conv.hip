@@ -11,14 +11,7 @@ namespace scn {
 
 bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* ranges, const uint16_t* bias_fp16,
                        int prec) {
-  cout = shape[0];
-  ks[0] = shape[1];
-  ks[1] = shape[2];
-  ks[2] = shape[3];
-  cin = shape[4];
-  kvol = ks[0] * ks[1] * ks[2];
-  precision = prec;
-  if (cout <= 0 || cin <= 0 || kvol <= 0) {
+  if (!set_geometry(shape, prec)) {
     set_error("invalid weight shape");
     return false;
   }
@@ -27,13 +20,6 @@ bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* 
     return false;
   }
   const int epc = prec == SCN_PRECISION_INT8 ? 16 : 8;  // elements per 16-byte chunk
-  int ch = (cin + epc - 1) / epc;
-  int p2 = 1;
-  while (p2 < ch) p2 <<= 1;  // chunks per row rounded to a power of two (rows are padded to it)
-  chunks = p2;
-  cin_pad = (uint32_t)(chunks * epc);
-  mtiles = (cout + 15) / 16;
-  steps = (kvol * chunks + 3) / 4;
   const int cout_pad = mtiles * 16;
   std::vector<float> ws(cout_pad, 1.f), bs(cout_pad, 0.f);
   for (int c = 0; c < cout; ++c) {
@@ -67,9 +53,6 @@ bool ConvWeights::init(const uint16_t* w_fp16, const int shape[5], const float* 
   // 32x32 MFMA order for layers with more than 16 output channels: [step][mtile32][lane] x 16 bytes,
   // lane l = channel 32 t + l % 32, K-half l / 32; K-step s holds chunks 2s, 2s+1 of the sequence
   if (mtiles >= 1) {
-    mtiles32 = (cout + 31) / 32;
-    if (mtiles32 == 3) mtiles32 = 4;  // kernels exist for 1, 2 and 4 tiles; the fourth is zero weights
-    steps32 = 4 * ((kvol * chunks + 7) / 8);  // whole iterations of 4 K-steps, zero weights beyond the volume
     std::vector<uint8_t> f32((size_t)steps32 * mtiles32 * 64 * 16, 0);
     for (int s = 0; s < steps32; ++s)
       for (int t = 0; t < mtiles32; ++t)
@@ -246,8 +229,10 @@ int scn_conv_forward(const scn_conv* c, const scn_rulebook* rb, const scn_conv_i
       pv.nbr = tp.nbr.as<int32_t>();
     }
   }
-  return conv_forward(c->w, rb->rb.nbr.as<int32_t>(), rb->rb.ld, rb->rb.n_out_dev(), rb->rb.n_bound_out,
-                      rb->rb.n_out_hint(), *io, (hipStream_t)stream, tp.built ? &pv : nullptr);
+  int rc = conv_forward(c->w, rb->rb.nbr.as<int32_t>(), rb->rb.ld, rb->rb.n_out_dev(), rb->rb.n_bound_out,
+                        rb->rb.n_out_hint(), *io, (hipStream_t)stream, tp.built ? &pv : nullptr);
+  if (rc == SCN_OK && debug_sync_enabled()) rc = debug_sync_check((hipStream_t)stream, "scn_conv_forward");
+  return rc;
 }
 
 }  // extern "C"

@@ -103,11 +103,14 @@ __device__ __forceinline__ bool coord_key(const int4 c, const Int3 g, uint32_t* 
 __global__ __launch_bounds__(256) void k_hash_insert(uint64_t* slots, uint32_t mask, const int4* __restrict__ coords,
                                                      uint32_t n_bound, const uint32_t* n_dev, Int3 grid,
                                                      uint32_t* n_eff_out, uint32_t* filter,
-                                                     const uint32_t* skip_if_zero) {
+                                                     const uint32_t* skip_if_zero, uint32_t* sorted_hint_host) {
   __shared__ uint32_t akeys[kAggSlots], avals[kAggSlots];
   const uint32_t r = blockIdx.x * blockDim.x + threadIdx.x;
   // (the flag first: a grid that only has to leave should not wait for the row count as well)
   const bool skip = skip_if_zero && *skip_if_zero == 0;
+  // pinned host word: 1 when this build found the rows in canonical order, 0 when it did not or did not look.  The host
+  // reads it when it enqueues a later build (a launch hint only, possibly one build behind).
+  if (r == 0 && sorted_hint_host) *sorted_hint_host = skip ? 1u : 0u;
   if (skip && !(r == 0 && n_eff_out)) return;
   const uint32_t n = eff_n(n_dev, n_bound);
   if (r == 0 && n_eff_out) {
@@ -247,7 +250,8 @@ int hash_build(const CoordTable& t, const int32_t* idx, uint32_t n, const uint32
                        t.filter.as<uint32_t>(), t.first_row.as<uint32_t>(), t.unsorted_flag());
   hipLaunchKernelGGL(k_hash_insert, dim3(blocks), dim3(256), 0, stream, t.slots(), t.mask,
                      (const int4*)idx, n, n_dev, g, n_eff_out, t.filter_words ? t.filter.as<uint32_t>() : nullptr,
-                     tm.probed ? (const uint32_t*)t.unsorted_flag() : (const uint32_t*)nullptr);
+                     tm.probed ? (const uint32_t*)t.unsorted_flag() : (const uint32_t*)nullptr,
+                     t.sorted_hint.as<uint32_t>());
   SCN_HIP(hipGetLastError());
   return SCN_OK;
 }
@@ -422,7 +426,6 @@ __global__ __launch_bounds__(256) void k_build_nbr(const int4* __restrict__ out_
       n_publish[1] = n;
     }
     if (n_host) *n_host = n;  // pinned host word: the row count as a launch hint for the next forward
-    if (lk.sorted_hint_host) *lk.sorted_hint_host = by_rank ? 1u : 0u;
   }
   const int k01 = blockIdx.y;  // k0 * K1 + k1
   if (o >= n) {
@@ -604,7 +607,6 @@ CoordLookup CoordTable::lookup() const {
     lk.unsorted = unsorted_flag();
     lk.first_row = first_row.as<uint32_t>();
   }
-  lk.sorted_hint_host = sorted_hint.as<uint32_t>();   // (the consumer records 0 when the build did not look)
   return lk;
 }
 
@@ -619,6 +621,7 @@ CoordLookup Rulebook::out_lookup() const {
 int Rulebook::build_subm(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3], const int ks[3],
                          const int dil[3], const CoordLookup* shared_lookup, hipStream_t stream) {
   const int one[3] = {1, 1, 1};
+  plan.built = false;   // a tile plan describes the table of one build
   int rc = check_geom(ks, one, dil, kvol_cap);
   if (rc) return rc;
   SCN_REQUIRE(n <= max_in && n <= ld, SCN_ERR_CAPACITY, "submanifold rulebook: %u rows exceed capacity %u", n, max_in);
@@ -680,6 +683,7 @@ int Rulebook::reserve_subm(bool need_own_in_table) {
 int Rulebook::build_sparse(const int32_t* idx, uint32_t n, const uint32_t* n_dev, const int grid[3], const int ks[3],
                            const int stride[3], const int pad[3], const int dil[3],
                            const CoordLookup* shared_lookup, hipStream_t stream) {
+  plan.built = false;   // a tile plan describes the table of one build
   int rc = check_geom(ks, stride, dil, kvol_cap);
   if (rc) return rc;
   SCN_REQUIRE(n <= max_in, SCN_ERR_CAPACITY, "sparse rulebook: %u rows exceed capacity %u", n, max_in);
@@ -809,6 +813,7 @@ __global__ __launch_bounds__(256) void k_fill_table_rows(int32_t* table, uint32_
 }
 
 int Rulebook::build_inverse(const Rulebook& fwd, const uint32_t* n_in_dev, hipStream_t stream) {
+  plan.built = false;   // a tile plan describes the table of one build
   SCN_REQUIRE(fwd.built && !fwd.subm, SCN_ERR_INVALID, "inverse rulebook: needs a built strided rulebook");
   SCN_REQUIRE(fwd.geom.kvol <= kvol_cap, SCN_ERR_CAPACITY, "inverse rulebook: kernel volume %d exceeds %d",
               fwd.geom.kvol, kvol_cap);
@@ -1019,7 +1024,7 @@ int scn_hash_build(uint64_t* table_dev, size_t capacity, const int32_t* indices_
   if (n) {
     hipLaunchKernelGGL(k_hash_insert, dim3(ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, table_dev,
                        (uint32_t)(capacity - 1), (const int4*)indices_dev, n, n_dev, g, (uint32_t*)nullptr,
-                       (uint32_t*)nullptr, (const uint32_t*)nullptr);
+                       (uint32_t*)nullptr, (const uint32_t*)nullptr, (uint32_t*)nullptr);
     SCN_HIP(hipGetLastError());
   }
   return SCN_OK;
@@ -1146,6 +1151,7 @@ int scn_voxelizer_forward_points(scn_voxelizer* v, const void* points_fp16_dev, 
                          v->counts.as<uint32_t>(), v->mins.as<uint32_t>(), (_Float16*)v->feats.p);
   }
   SCN_HIP(hipGetLastError());
+  if (debug_sync_enabled()) return debug_sync_check(stream, "scn_voxelizer_forward");
   return SCN_OK;
 }
 
@@ -1189,19 +1195,25 @@ void scn_rulebook_destroy(scn_rulebook* rb) { delete rb; }
 int scn_rulebook_build_subm(scn_rulebook* rb, const int32_t* indices_dev, uint32_t n, const uint32_t* n_dev,
                             const int grid[3], const int ksize[3], const int dilation[3], void* stream) {
   SCN_REQUIRE(rb && grid && ksize && dilation && (indices_dev || n == 0), SCN_ERR_INVALID, "null pointer");
-  return rb->rb.build_subm(indices_dev, n, n_dev, grid, ksize, dilation, nullptr, (hipStream_t)stream);
+  int rc = rb->rb.build_subm(indices_dev, n, n_dev, grid, ksize, dilation, nullptr, (hipStream_t)stream);
+  if (rc == SCN_OK && debug_sync_enabled()) rc = debug_sync_check((hipStream_t)stream, "scn_rulebook_build_subm");
+  return rc;
 }
 int scn_rulebook_build_sparse(scn_rulebook* rb, const int32_t* indices_dev, uint32_t n, const uint32_t* n_dev,
                               const int grid[3], const int ksize[3], const int stride[3], const int padding[3],
                               const int dilation[3], void* stream) {
   SCN_REQUIRE(rb && grid && ksize && stride && padding && dilation && (indices_dev || n == 0), SCN_ERR_INVALID,
               "null pointer");
-  return rb->rb.build_sparse(indices_dev, n, n_dev, grid, ksize, stride, padding, dilation, nullptr,
-                             (hipStream_t)stream);
+  int rc = rb->rb.build_sparse(indices_dev, n, n_dev, grid, ksize, stride, padding, dilation, nullptr,
+                               (hipStream_t)stream);
+  if (rc == SCN_OK && debug_sync_enabled()) rc = debug_sync_check((hipStream_t)stream, "scn_rulebook_build_sparse");
+  return rc;
 }
 int scn_rulebook_build_inverse(scn_rulebook* rb, const scn_rulebook* forward, const uint32_t* n_in_dev, void* stream) {
   SCN_REQUIRE(rb && forward, SCN_ERR_INVALID, "null pointer");
-  return rb->rb.build_inverse(forward->rb, n_in_dev, (hipStream_t)stream);
+  int rc = rb->rb.build_inverse(forward->rb, n_in_dev, (hipStream_t)stream);
+  if (rc == SCN_OK && debug_sync_enabled()) rc = debug_sync_check((hipStream_t)stream, "scn_rulebook_build_inverse");
+  return rc;
 }
 const int32_t* scn_rulebook_nbr(const scn_rulebook* rb) { return rb ? rb->rb.nbr.as<int32_t>() : nullptr; }
 uint32_t scn_rulebook_nbr_ld(const scn_rulebook* rb) { return rb ? rb->rb.ld : 0; }

@@ -123,6 +123,8 @@ struct RtTensor {
   bool fixed_form = false;     // dense tensor in a vectorised layout: a following Reshape keeps this shape
   int view_of = -1;    // dense view of another tensor (reshape / fused transpose)
   bool materialised = false;  // false: fused away, never written
+  bool shared = false;        // storage shared with tensors of disjoint lifetimes: holds this tensor's values only
+                              // between the step that writes it and the last step that reads it
 };
 
 enum class StepKind { InputCount, HashBuild, RulebookSubm, RulebookSparse, RulebookInverse, Convert, Conv, Add, Relu, Dense, Permute };
@@ -948,7 +950,8 @@ static int allocate_runtime(scn_engine& e) {
       x.data = x.buf.p;
       continue;
     }
-    if (slot_of[t] >= 0) {
+    x.shared = slot_of[t] >= 0;
+    if (x.shared) {
       x.buf.release();
       x.data = e.arena[slot_of[t]].p;
       continue;
@@ -1577,6 +1580,9 @@ static std::vector<int> attr_ints3(const OnnxNode& n, const char* name) {
   return out;
 }
 
+static scn_engine* create_from_model_bytes(const std::string& bytes, const char* onnx_file, int precision, unsigned flags,
+                                           unsigned fixed_launch_points, const scn_load_options* options, void* stream);
+
 scn_engine* scn_engine_create_from_onnx(const char* onnx_file, int precision, unsigned flags,
                                         unsigned fixed_launch_points, void* stream) {
   return scn_engine_create_from_onnx_ex(onnx_file, precision, flags, fixed_launch_points, nullptr, stream);
@@ -1586,6 +1592,29 @@ scn_engine* scn_engine_create_from_onnx_ex(const char* onnx_file, int precision,
                                            unsigned fixed_launch_points, const scn_load_options* options,
                                            void* stream) {
   if (!onnx_file) return nullptr;
+  SCN_LOGV("Load onnx from: %s", onnx_file);
+  std::ifstream fin(onnx_file, std::ios::binary);
+  if (!fin) {
+    set_error("Parse onnx failed: %s (cannot open)", onnx_file);
+    return nullptr;
+  }
+  const std::string bytes((std::istreambuf_iterator<char>(fin)), std::istreambuf_iterator<char>());
+  return create_from_model_bytes(bytes, onnx_file, precision, flags, fixed_launch_points, options, stream);
+}
+
+scn_engine* scn_engine_create_from_onnx_memory(const void* model_bytes, size_t size, int precision, unsigned flags,
+                                               unsigned fixed_launch_points, const scn_load_options* options,
+                                               void* stream) {
+  if (!model_bytes && size) {
+    set_error("create_from_onnx_memory: null model");
+    return nullptr;
+  }
+  const std::string bytes(static_cast<const char*>(model_bytes), size);
+  return create_from_model_bytes(bytes, "(memory)", precision, flags, fixed_launch_points, options, stream);
+}
+
+static scn_engine* create_from_model_bytes(const std::string& bytes, const char* onnx_file, int precision, unsigned flags,
+                                           unsigned fixed_launch_points, const scn_load_options* options, void* stream) {
   const scn_precision_override* overrides = options ? options->overrides : nullptr;
   const int n_overrides = options ? options->n_overrides : 0;
   const scn_tensor_amax* ranges = options ? options->ranges : nullptr;
@@ -1601,13 +1630,6 @@ scn_engine* scn_engine_create_from_onnx_ex(const char* onnx_file, int precision,
       if (ranges[i].tensor && tensor == ranges[i].tensor) r = ranges[i].amax;
     return r;
   };
-  SCN_LOGV("Load onnx from: %s", onnx_file);
-  std::ifstream fin(onnx_file, std::ios::binary);
-  if (!fin) {
-    set_error("Parse onnx failed: %s (cannot open)", onnx_file);
-    return nullptr;
-  }
-  std::string bytes((std::istreambuf_iterator<char>(fin)), std::istreambuf_iterator<char>());
   OnnxGraph g;
   if (bytes.empty() || !parse_model(bytes, g)) {
     set_error("Parse onnx failed: %s", onnx_file);
@@ -1629,8 +1651,17 @@ scn_engine* scn_engine_create_from_onnx_ex(const char* onnx_file, int precision,
         }
         size_t vol = 1;
         shape.clear();
-        for (auto d : t.dims) { shape.push_back((int)d); vol *= (size_t)d; }
-        if (vol * 2 != t.raw.size()) {
+        for (auto d : t.dims) {
+          // (each dimension and the volume stay far inside int and size_t, so that the builder's own products of
+          // the int shape cannot differ from this one)
+          if (d < 1 || d > (1 << 24) || vol > ((size_t)1 << 31) / (size_t)d) {
+            set_error("Invalid dimensions of initializer '%s'.", name.c_str());
+            return false;
+          }
+          shape.push_back((int)d);
+          vol *= (size_t)d;
+        }
+        if (t.dims.empty() || vol * 2 != t.raw.size()) {
           set_error("Invalid parameter data size. %zu != %zu", vol * 2, t.raw.size());
           return false;
         }
@@ -1817,7 +1848,8 @@ int scn_engine_forward(scn_engine* e, void* stream_) {
   // stream first, in graph order, and runs as far ahead of the feature kernels as the GPU allows; the
   // main stream then waits per rulebook.  The auxiliary stream is in order, so waiting for a rulebook's
   // event also covers everything built before it.
-  const bool dual = e->aux != nullptr && !e->profiling;
+  const bool debug = debug_sync_enabled();
+  const bool dual = e->aux != nullptr && !e->profiling && !debug;
   auto is_coord_step = [](const Step& st) {
     return st.kind == StepKind::HashBuild || st.kind == StepKind::RulebookSubm || st.kind == StepKind::RulebookSparse ||
            st.kind == StepKind::RulebookInverse;
@@ -1929,6 +1961,7 @@ int scn_engine_forward(scn_engine* e, void* stream_) {
       SCN_HIP(hipEventRecord(st.ev0, stream));
     }
     int rc = run_step(*e, st, stream);
+    if (rc == SCN_OK && debug) rc = debug_sync_check(stream, st.label.c_str());
     if (rc) return fail(st, rc);
     if (e->profiling) SCN_HIP(hipEventRecord(st.ev1, stream));
   }
@@ -1972,6 +2005,10 @@ int scn_engine_tensor(scn_engine* e, const char* name, scn_tensor_view* view, vo
   SCN_REQUIRE(it != e->tensor_by_name.end(), SCN_ERR_INVALID, "tensor '%s' does not exist", name);
   SCN_REQUIRE(e->tensors[it->second].materialised, SCN_ERR_INVALID,
               "tensor '%s' was fused away (build with SCN_BUILD_KEEP_ALL to keep it)", name);
+  // (decided by allocate_runtime; before the first forward / prepare nothing is shared yet, and nothing holds values)
+  SCN_REQUIRE(!e->tensors[it->second].shared, SCN_ERR_INVALID,
+              "tensor '%s' shares its storage with other intermediate tensors and does not hold its values after a "
+              "forward (build with SCN_BUILD_KEEP_ALL to keep it, or make it a graph output)", name);
   fill_view(e, it->second, view);
   if (acc_dev) *acc_dev = e->tensors[it->second].acc.p;
   return SCN_OK;
@@ -1986,7 +2023,7 @@ int scn_engine_collect_amax(scn_engine* e, void* stream_, scn_tensor_amax* out, 
   std::vector<int> which;
   for (size_t t = 0; t < e->tdesc.size() && t < e->tensors.size(); ++t) {
     const RtTensor& x = e->tensors[t];
-    if (x.dense || x.coord < 0 || !x.materialised) continue;
+    if (x.dense || x.coord < 0 || !x.materialised || x.shared) continue;   // (shared storage holds another tensor's bytes by now)
     if ((int)t == e->inputs[0] ? e->in_feat == nullptr : x.data == nullptr) continue;
     which.push_back((int)t);
   }

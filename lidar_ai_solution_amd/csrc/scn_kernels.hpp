@@ -22,7 +22,6 @@ struct CoordLookup {
   // of the word's lowest set bit, so a look-up is a rank (two loads) and the hash table was not filled at all.
   const uint32_t* unsorted = nullptr;
   const uint32_t* first_row = nullptr;
-  uint32_t* sorted_hint_host = nullptr;  // pinned host word: 1 when the last build that has run found canonical order
 };
 
 struct CoordTable {
@@ -136,6 +135,29 @@ struct ConvWeights {
   DevBuf wscale;    // fp32 [cout_pad]: s_w[c] (int8) or 1
   DevBuf bias;      // fp32 [cout_pad]
   bool init(const uint16_t* w_fp16, const int shape[5], const float* ranges, const uint16_t* bias_fp16, int prec);
+  // the sizes above from a weight shape [Cout, K0, K1, K2, Cin] (host only; false for a shape with a dimension < 1)
+  bool set_geometry(const int shape[5], int prec) {
+    cout = shape[0];
+    ks[0] = shape[1];
+    ks[1] = shape[2];
+    ks[2] = shape[3];
+    cin = shape[4];
+    if (cout <= 0 || cin <= 0 || ks[0] <= 0 || ks[1] <= 0 || ks[2] <= 0) return false;
+    kvol = ks[0] * ks[1] * ks[2];
+    precision = prec;
+    const int epc = prec == SCN_PRECISION_INT8 ? 16 : 8;  // elements per 16-byte chunk
+    const int ch = (cin + epc - 1) / epc;
+    int p2 = 1;
+    while (p2 < ch) p2 <<= 1;  // chunks per row rounded to a power of two (rows are padded to it)
+    chunks = p2;
+    cin_pad = (uint32_t)(chunks * epc);
+    mtiles = (cout + 15) / 16;
+    steps = (kvol * chunks + 3) / 4;
+    mtiles32 = (cout + 31) / 32;
+    if (mtiles32 == 3) mtiles32 = 4;  // kernels exist for 1, 2 and 4 tiles; the fourth is zero weights
+    steps32 = 4 * ((kvol * chunks + 7) / 8);  // whole iterations of 4 K-steps, zero weights beyond the volume
+    return true;
+  }
 };
 
 // n_hint: expected row count (0 = unknown), only used to choose the launch configuration

@@ -40,7 +40,8 @@ from typing import Dict, List, Optional, Tuple
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "libscn_oracle.so")
+# SCN_ORACLE_LIB names another build of the same source (the sanitizer build of the Makefile's `sanitize` target)
+_LIB_PATH = os.environ.get("SCN_ORACLE_LIB") or os.path.join(_HERE, "libscn_oracle.so")
 _lib = None
 
 

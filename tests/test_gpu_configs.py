@@ -58,13 +58,43 @@ def test_config2_fp16_backbone_full_size(frame250k):
     assert maxabs <= FP16_REL * refmax and cos >= FP16_COS
 
 
-def test_config3_int8_backbone_full_size_and_row_order_invariance(frame250k):
+def _voxelize_zyx(points):
+    return _voxelize_gpu(points, "zyx")
+
+
+@pytest.fixture(scope="module")
+def headline_int8_models(frame250k):
+    """The benchmark's own int8 model (lidar_ai_solution_amd/workload.py: seeded weights, ranges calibrated on the four
+    seeded calibration frames with the fp16 engine) at the two row capacities: the exporters' default, which cuts
+    stage 1 of this frame at 200,000 rows, and the benchmark's 400,000, which cuts nothing."""
+    from lidar_ai_solution_amd import workload
+    frames = [_voxelize_zyx(synth.lidar_frame(seed=s, n_points=250000)) for s in workload.CALIBRATION_SEEDS]
+    return {b: workload.headline_model("int8", _voxelize_zyx, output_bound=b, calibration_frames=frames)
+            for b in (200000, workload.OUTPUT_BOUND)}
+
+
+def _library_source_hash():
+    import glob, hashlib, os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    h = hashlib.sha256()
+    for path in sorted(glob.glob(os.path.join(root, "lidar_ai_solution_amd", "csrc", "*"))):
+        with open(path, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+@pytest.mark.parametrize("bound", [200000, 400000])
+def test_config3_int8_backbone_full_size_and_row_order_invariance(bound, frame250k, headline_int8_models):
+    """Every int8 accumulator, every stored tensor and the BEV output of the benchmark's model, bit for bit, at the
+    truncating default output_bound and at the benchmark's own (stages of 322,224 / 214,656 / 68,948 / 64,790 rows:
+    the launch shapes of the headline figure).  The CRC-32 of the BEV bytes is printed and recorded; bench.py prints
+    the same checksum of its output next to the recorded one."""
+    import json, os
+    from lidar_ai_solution_amd import workload
     f, i = frame250k
-    note(f"config 3: int8 CenterPoint-shaped backbone, {f.shape[0]} voxels, default output_bound (stage 1 truncates)")
-    g16, tags = graphs.centerpoint_scn(seed=0)
-    amax = _oracle_calibration(g16, f, i, GRID_ZYX)
-    g8, tags8 = graphs.centerpoint_scn(seed=0)
-    graphs.apply_int8_plan(g8, tags8, amax, "centerpoint")
+    g8 = headline_int8_models[bound]
+    note(f"config 3: int8 CenterPoint-shaped backbone, {f.shape[0]} voxels, output_bound {bound}"
+         f"{' (stage 1 truncates)' if bound == 200000 else ' (the benchmark workload, nothing truncated)'}")
     keep = Engine.from_graph(g8, "int8", keep_all=True)
     _run_engine(keep, f, i, GRID_ZYX)
     rec = _oracle_walk_rebased(g8, keep, f, i, GRID_ZYX)
@@ -75,6 +105,7 @@ def test_config3_int8_backbone_full_size_and_row_order_invariance(frame250k):
     hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
     prec = O.node_precisions(g8, "int8")
     nconv = 0
+    rows = []
     for n in g8.nodes:
         if n.op_type == "SparseConvolution" and prec[n.name][0] == "int8":
             view, acc_ptr = keep.tensor(n.outputs[0])
@@ -86,11 +117,35 @@ def test_config3_int8_backbone_full_size_and_row_order_invariance(frame250k):
             feats, _ = view.torch()
             assert np.array_equal(feats.cpu().numpy()[:, :a.shape[1]], rec[n.name]["out"]), n.name
             nconv += 1
+            if not n.attrs.get("subm"):
+                rows.append(a.shape[0])
     assert nconv == 18
-    eng = Engine.from_graph(g8, "int8")
-    _run_engine(eng, f, i, GRID_ZYX)
-    got = eng.output(0).torch().cpu().numpy()
-    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    if bound == 400000:
+        assert rows == [322224, 214656, 68948, 64790], rows      # nothing truncated: the benchmark's stage sizes
+    else:
+        assert rows[0] == 200000, rows
+    keep.close()
+    for aux in (False, True):
+        eng = Engine.from_graph(g8, "int8", with_auxiliary_stream=aux)
+        _run_engine(eng, f, i, GRID_ZYX)
+        got = eng.output(0).torch().cpu().numpy()
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), f"fused engine, auxiliary stream {aux}"
+    crc = workload.bev_checksum(got)
+    assert crc == workload.bev_checksum(want)
+    print(f"config 3 BEV checksum (CRC-32 of the output bytes, output_bound {bound}): {crc}")
+    if bound == 400000:
+        root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+        record = {"precision": "int8", "points": 250000, "active_voxels": int(f.shape[0]), "output_bound": bound,
+                  "library_sources": _library_source_hash(), "crc32": crc}
+        os.makedirs(os.path.join(root, "gpurun_out"), exist_ok=True)
+        with open(os.path.join(root, "gpurun_out", "headline_bev_checksum.json"), "w") as fh:
+            json.dump({"records": [record]}, fh, indent=1)
+        golden = os.path.join(root, "tests", "golden", "headline_bev_checksum.json")
+        if os.path.exists(golden):
+            with open(golden) as fh:
+                for r in json.load(fh).get("records", []):
+                    if all(r.get(k) == v for k, v in record.items() if k != "crc32"):
+                        assert r["crc32"] == crc, "the recorded checksum claims these library sources and differs"
     note("property: the dense output does not depend on the order of the input rows (int8 path, bit for bit)")
     perm = np.random.default_rng(1).permutation(f.shape[0])
     _run_engine(eng, f[perm], i[perm], GRID_ZYX)

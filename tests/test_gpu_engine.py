@@ -854,3 +854,108 @@ def test_cpp_centerpoint_preprocessing_and_legacy_engine_on_a_raw_fp32_sweep(cp_
     got = tensor.load(prefix + ".bev.tensor")
     assert got.shape == (1, 256, 180, 180)
     assert np.array_equal(got.view(np.uint16), eng.output(0).torch().cpu().numpy().view(np.uint16))
+
+
+def _three_output_model(feats, idx):
+    """All-int8 CenterPoint-shaped graph with three outputs (README.md:14-19 of the reference's library: "Multiple
+    outputs are supported"; engine.hpp:72-75 num_output / output(i)): the dense BEV, the int8 sparse tensor that ends a
+    block (the next block's convolution input AND the residual operand of its fused Conv + Add + ReLU), and the second
+    convolution of a block, which would otherwise be fused into the Add behind it."""
+    g16, _ = graphs.centerpoint_scn(seed=4)
+    amax = _oracle_calibration(g16, feats, idx, GRID_ZYX)
+    g8, tags8 = graphs.centerpoint_scn(seed=4)
+    graphs.apply_int8_plan(g8, tags8, amax, "all-int8")
+    relus = [n for n in g8.nodes if n.op_type == "Relu"]
+    adds = [n for n in g8.nodes if n.op_type == "Add"]
+    block_end = relus[2].outputs[0]          # end of the first 32-channel block: read by a conv and by an Add
+    conv2 = adds[4].inputs[0]                # second convolution of the first 64-channel block
+    assert [n.op_type for n in g8.nodes if block_end in n.inputs] == ["SparseConvolution", "Add"]
+    g8.outputs = [g8.outputs[0], block_end, conv2]
+    return g8
+
+
+@pytest.mark.parametrize("rows", [79745, 25000])
+def test_graph_with_three_outputs_dense_and_intermediate_sparse(rows, centerpoint_input, tmp_path):
+    feats, idx = centerpoint_input
+    feats, idx = feats[:rows], idx[:rows]
+    g8 = _three_output_model(feats, idx)
+    want = O.run_graph(g8, feats, idx, GRID_ZYX, "int8")
+    path = str(tmp_path / "three_outputs.scn.onnx")
+    onnx_dialect.save(g8, path)
+    assert onnx_dialect.load(path).outputs == g8.outputs
+
+    def check(eng, what):
+        assert eng.num_output() == 3, what
+        dense = eng.output(0)
+        assert dense.dense and np.array_equal(dense.torch().cpu().numpy().view(np.uint16), want[g8.outputs[0]].view(np.uint16)), what
+        for k in (1, 2):
+            v = eng.output(k)
+            w = want[g8.outputs[k]]
+            assert not v.dense and v.name == g8.outputs[k] and v.dtype == capi.DTYPE_INT8, (what, k)
+            assert np.float32(v.dynamic_range) == np.float32(w.rng), (what, k)
+            f, i = v.torch()
+            assert v.num_rows() == w.feat.shape[0] and v.grid_size == list(w.grid), (what, k)
+            assert np.array_equal(i.cpu().numpy(), w.indices), (what, k)
+            assert np.array_equal(f.cpu().numpy()[:, :w.feat.shape[1]], w.feat), f"{what}: sparse output {k}"
+
+    n_steps = {}
+    for what, make in (("fused, one stream", lambda: Engine.from_graph(g8, "int8")),
+                       ("fused, auxiliary stream", lambda: Engine.from_graph(g8, "int8", with_auxiliary_stream=True)),
+                       ("every tensor kept", lambda: Engine.from_graph(g8, "int8", keep_all=True)),
+                       ("loaded from the model file", lambda: Engine.from_onnx(path, "int8")),
+                       ("sortmask", lambda: Engine.from_graph(g8, "int8", sortmask=True))):
+        note(f"three-output int8 graph on {rows} rows: {what}")
+        eng = make()
+        _run_engine(eng, feats, idx, GRID_ZYX)
+        check(eng, what)
+        _run_engine(eng, feats[:rows // 2], idx[:rows // 2], GRID_ZYX)      # outputs own their storage: a second,
+        _run_engine(eng, feats, idx, GRID_ZYX)                              # smaller frame leaves nothing behind
+        check(eng, what + ", third forward")
+        n_steps[what] = len(eng.step_times())
+        eng.close()
+    # the other blocks are still fused in the engine that is allowed to fuse
+    assert n_steps["fused, one stream"] < n_steps["every tensor kept"] - 8, n_steps
+    # the same model with one output gives the same dense tensor (an extra output changes no arithmetic)
+    g1 = _three_output_model(feats, idx)
+    g1.outputs = g1.outputs[:1]
+    e1 = Engine.from_graph(g1, "int8")
+    _run_engine(e1, feats, idx, GRID_ZYX)
+    assert np.array_equal(e1.output(0).torch().cpu().numpy().view(np.uint16), want[g8.outputs[0]].view(np.uint16))
+
+
+def test_intermediate_tensors_with_shared_storage_are_not_handed_out(cp_models, centerpoint_input):
+    """Without SCN_BUILD_KEEP_ALL the intermediate sparse tensors share storage by lifetime: after a forward such a
+    tensor's bytes belong to a later tensor.  scn_engine_tensor refuses them by name, scn_engine_collect_amax leaves them
+    out, and what both still report equals the keep-all engine's."""
+    feats, idx = centerpoint_input
+    n = 30000
+    feats, idx = feats[:n], idx[:n]
+    g16, _ = cp_models
+    keep = Engine.from_graph(g16, "fp16", keep_all=True)
+    eng = Engine.from_graph(g16, "fp16")
+    _run_engine(keep, feats, idx, GRID_ZYX)
+    _run_engine(eng, feats, idx, GRID_ZYX)
+    all_amax = keep.collect_amax()
+    some = eng.collect_amax()
+    note(f"engine without keep-all reports {len(some)} of {len(all_amax)} tensors")
+    assert g16.inputs[0] in some and 1 <= len(some) < len(all_amax)
+    for name, v in some.items():
+        assert np.float32(v) == np.float32(all_amax[name]), name
+    refused = handed = 0
+    for nd in g16.nodes:
+        if nd.op_type not in ("SparseConvolution", "Add", "Relu"):
+            continue
+        name = nd.outputs[0]
+        try:
+            view, _ = eng.tensor(name)
+        except RuntimeError as e:
+            assert "fused away" in str(e) or "shares its storage" in str(e), str(e)
+            assert name not in some
+            refused += 1
+            continue
+        assert name in some, name          # handed out = owns its storage = reported
+        f, _ = view.torch()
+        kf, _ = keep.tensor(name)[0].torch()
+        assert torch.equal(f.view(torch.int16), kf.view(torch.int16)), name
+        handed += 1
+    assert refused >= 20, (refused, handed)

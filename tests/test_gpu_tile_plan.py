@@ -117,6 +117,9 @@ def test_conv_with_plan_equals_conv_without(cin, cout, strided, el, centerpoint_
         want16 = O.epilogue(acc_ref, scale, b.astype(np.float32), False, False)
         res = rng.integers(-127, 128, (n_out, (cout + 15) // 16 * 16)).astype(np.int8)
         d_x, d_res = to_dev(x), to_dev(res)
+        # the fused Conv + Add + ReLU of the un-fused oracle: int8 intermediate, int8 add, ReLU, int8 store
+        mid = O.epilogue(acc_ref, scale, b.astype(np.float32), False, True, 1.7)
+        want_fused = O.add(mid, 1.7, res[:, :cout], 2.2, True, True, out_range)
         results = []
         for plan in (None, 0, 1):
             if plan is not None:
@@ -131,7 +134,7 @@ def test_conv_with_plan_equals_conv_without(cin, cout, strided, el, centerpoint_
             assert np.array_equal(r[1], acc_ref), f"accumulators, variant {k}"
             assert np.array_equal(r[0][:, :cout], want8) and np.array_equal(r[2][:, :cout], want8), f"int8 output, variant {k}"
             assert np.array_equal(r[3][:, :cout].view(np.uint16), want16.view(np.uint16)), f"fp16 output, variant {k}"
-            assert np.array_equal(r[4], results[0][4]), f"fused residual, variant {k}"
+            assert np.array_equal(r[4][:, :cout], want_fused), f"fused residual against the un-fused oracle, variant {k}"
         assert np.count_nonzero(results[0][4]) > n_out
     else:
         cpad = 8 if cin == 5 else cin
@@ -149,15 +152,46 @@ def test_conv_with_plan_equals_conv_without(cin, cout, strided, el, centerpoint_
                 capi.check(L.scn_rulebook_build_plan(rb.h, plan, stream()))
             o, _ = conv.forward(rb, d_x, n_out, relu=True, out_int8=False)
             f, _ = conv.forward(rb, d_x, n_out, relu=False, out_int8=False, res=d_res, relu2=True)
-            outs.append((o.cpu().numpy(), f.cpu().numpy()))
+            m, _ = conv.forward(rb, d_x, n_out, relu=False, out_int8=False)
+            outs.append((o.cpu().numpy(), f.cpu().numpy(), m.cpu().numpy()))
         tol = 2e-3 * max(float(np.abs(want).max()), 1e-3)   # a few fp16 steps of the largest value: products are summed in fp32
-        for k, (o, f) in enumerate(outs):
+        for k, (o, f, m) in enumerate(outs):
             assert np.abs(o[:, :cout].astype(np.float32) - want).max() <= tol, f"variant {k}"
+            # fused fp16 Conv + Add + ReLU, exactly: the oracle's Add of the same kernel's un-fused fp16 result (same MFMA
+            # sequence, no ReLU) and the residual
+            want_f = O.add(np.ascontiguousarray(m[:, :cout]), 127.0, np.ascontiguousarray(res[:, :cout]), 127.0, True, False)
+            assert np.array_equal(f[:, :cout].view(np.uint16), want_f.view(np.uint16)), f"fused fp16 residual, variant {k}"
         # the sorted plan and the plan in row order add a row's products in the same order
         assert np.array_equal(outs[1][0].view(np.uint16), outs[2][0].view(np.uint16))
         assert np.array_equal(outs[1][1].view(np.uint16), outs[2][1].view(np.uint16))
         if cin != 5:   # rows of more than 16 bytes: the same MFMA sequence as the plan-less kernel, zero steps left out
             assert np.array_equal(outs[0][0].view(np.uint16), outs[1][0].view(np.uint16))
+
+
+def test_rebuilding_a_rulebook_drops_its_tile_plan():
+    """A plan describes the table of one build: after the rulebook is built again on other coordinates (without a new
+    plan) a convolution must not use the old masks, permutation or plan-order table."""
+    rng = np.random.default_rng(9)
+    L = capi.lib()
+    grid = (8, 64, 64)
+    idx_a = synth.uniform_voxels(6, 9000, grid)
+    idx_b = synth.uniform_voxels(7, 7001, grid)
+    w, b, ranges = _weights(rng, 32, (3, 3, 3), 32)
+    conv = GpuConv(w, ranges, b, capi.PRECISION_INT8)
+    wq, s_w = O.quantize_weights(w, ranges)
+    scale = (np.float32(2.0) / np.float32(127) * s_w).astype(np.float32)
+    rb = GpuRulebook(9000, 9000, 27)
+    for sorted_plan in (1, 0):
+        note(f"build -> plan (sorted={sorted_plan}) -> build on other coordinates -> convolution")
+        rb.build_subm(to_dev(idx_a), idx_a.shape[0], grid, (3, 3, 3))
+        capi.check(L.scn_rulebook_build_plan(rb.h, sorted_plan, stream()))
+        rb.build_subm(to_dev(idx_b), idx_b.shape[0], grid, (3, 3, 3))
+        assert L.scn_rulebook_plan(rb.h, None, None, None) != 0      # no plan any more
+        x = rng.integers(-127, 128, (idx_b.shape[0], 32)).astype(np.int8)
+        want = O.epilogue(O.conv_int8_acc(x, wq, O.rulebook_subm(idx_b, grid, (3, 3, 3))), scale, b.astype(np.float32),
+                          True, True, 1.5)
+        out, _ = conv.forward(rb, to_dev(x), idx_b.shape[0], x_range=2.0, relu=True, out_int8=True, out_range=1.5)
+        assert np.array_equal(out.cpu().numpy(), want)
 
 
 def test_plan_with_device_side_count_and_empty_input():
