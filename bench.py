@@ -58,6 +58,15 @@ def parse_args():
     ap.add_argument("--sortmask", dest="sortmask", action="store_true", default=False,
                     help="the reference loader's sortmask switch: rows of the narrow layers' rulebooks are sorted by "
                          "their sets of kernel offsets so that a tile visits few offsets (results are identical)")
+    ap.add_argument("--sweep", action="store_true",
+                    help="latency against frame size instead of the headline line: the eight density-gradient frames of "
+                         "BASELINE configuration 4 (50k - 300k points), the reference's nuScenes sweep and its 79,745-voxel "
+                         "demo input; per frame num_valid, voxelization_ms, scn_ms in int8 and fp16 (the three columns of "
+                         "the reference's perf log, libraries/3DSparseConvolution/workspace/perf-int8.log)")
+    ap.add_argument("--row-sweep", action="store_true",
+                    help="the dominant layer shape (int8 SubM 128->128, 3x3x3) alone on the coordinate sets of the four "
+                         "stages of the synthetic frame (68,948 .. 322,224 rows): us, TOP/s and fraction of the MFMA peak "
+                         "per size")
     ap.add_argument("--copy-probe", action="store_true",
                     help="first launch a plain copy kernel of known size (k_convert_rows fp16->fp16, 512 MiB read + "
                          "512 MiB written, 3 launches): the reference point that scales FETCH_SIZE / WRITE_SIZE counters")
@@ -253,6 +262,137 @@ def node_io_bytes(node, graph, precision, fused_add, n_out):
     return e, e_out, e, (n_out * cout * e_out if fused_add else 0)
 
 
+def time_forwards(eng, stream, reps=30, warm=5):
+    """ms per Engine.forward, direct launches, HIP events on the launch stream."""
+    import torch
+    with torch.cuda.stream(stream):
+        for _ in range(warm):
+            eng.forward()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            eng.forward()
+        e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def sweep(args):
+    """num_valid, voxelization_ms, scn_ms per frame (int8 and fp16 engines, weights and ranges of the headline model)."""
+    import torch
+    from lidar_ai_solution_amd import synth, workload
+    from lidar_ai_solution_amd.scn import Engine
+
+    def voxelize_np(points_np):
+        f_c, i_c, _, _, v_c = voxelize_on_gpu(points_np, "zyx")
+        v_c.close()
+        return f_c.cpu().numpy(), i_c.cpu().numpy()
+
+    frames = [(f"gradient frame {s}", synth.gradient_frame(seed=40 + s, n_points=npts))
+              for s, npts in enumerate([50000, 85000, 120000, 160000, 200000, 240000, 270000, 300000])]
+    golden = os.path.join(ROOT, "tests", "golden")
+    frames.append(("nuScenes sweep (reference demo)", np.load(os.path.join(golden, "nuscenes_frame.npz"))["points"]))
+    frames.append(("headline synthetic frame", workload.headline_points(args.points)))
+    graph8 = workload.headline_model("int8", voxelize_np, args.output_bound, args.points)
+    graph16 = workload.headline_model("fp16", voxelize_np, args.output_bound, args.points)
+    engines = {"int8": Engine.from_graph(graph8, "int8", with_auxiliary_stream=True),
+               "fp16": Engine.from_graph(graph16, "fp16", with_auxiliary_stream=True)}
+    stream = torch.cuda.Stream()
+    rows = []
+    inputs = []
+    for name, pts in frames:
+        feats, idx, nvox, vox_ms, vox = voxelize_on_gpu(pts, "zyx")
+        vox.close()
+        inputs.append((name, int(pts.shape[0]), feats, idx, nvox, vox_ms))
+    d = np.load(os.path.join(golden, "centerpoint_input.npz"))
+    inputs.append(("CenterPoint demo input (voxels given)", None,
+                   torch.from_numpy(np.ascontiguousarray(d["features"], dtype=np.float16)).cuda(),
+                   torch.from_numpy(np.ascontiguousarray(d["indices_zyx"], dtype=np.int32)).cuda(), int(d["indices_zyx"].shape[0]), None))
+    for name, npts, feats, idx, nvox, vox_ms in inputs:
+        row = {"frame": name, "points": npts, "num_valid": int(nvox), "voxelization_ms": None if vox_ms is None else round(vox_ms, 4)}
+        for prec, eng in engines.items():
+            eng.set_input(feats, idx, GRID_ZYX)
+            row[f"scn_ms_{prec}"] = round(time_forwards(eng, stream), 4)
+        rows.append(row)
+        print(row, file=sys.stderr, flush=True)
+    print(json.dumps({"metric": "latency against frame size, CenterPoint-shaped SCN backbone (secondary figures)",
+                      "launch": "direct launches, auxiliary stream", "output_bound": args.output_bound, "sweep": rows}))
+
+
+def row_sweep(args):
+    """The dominant layer shape on four row counts: the coordinate sets of the synthetic frame's stages."""
+    import torch
+    from lidar_ai_solution_amd import capi, workload
+    L = capi.lib()
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    feats, idx, nvox, _, vox = voxelize_on_gpu(workload.headline_points(args.points), "zyx")
+    vox.close()
+    geoms = [((3, 3, 3), (2, 2, 2), (1, 1, 1)), ((3, 3, 3), (2, 2, 2), (1, 1, 1)), ((3, 3, 3), (2, 2, 2), (0, 1, 1))]
+    sets = [(idx, int(nvox), list(GRID_ZYX))]
+    keep = []
+    for k, s_, p in geoms:
+        cur_idx, cur_n, cur_grid = sets[-1]
+        rb = L.scn_rulebook_create(cur_n, 400000, 27)
+        capi.check(L.scn_rulebook_build_sparse(rb, C.c_void_p(cur_idx.data_ptr()), cur_n, None, capi.i3(*cur_grid), capi.i3(*k),
+                                               capi.i3(*s_), capi.i3(*p), capi.i3(1, 1, 1), st))
+        torch.cuda.synchronize()
+        n_out_t = torch.empty(1, dtype=torch.int32, device="cuda")
+        hip = capi.hip_runtime()
+        hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        hip.hipMemcpy(C.c_void_p(n_out_t.data_ptr()), C.c_void_p(L.scn_rulebook_num_out_dev(rb)), 4, 3)
+        n_out = int(n_out_t.cpu().numpy()[0])
+        out_idx = torch.empty((n_out, 4), dtype=torch.int32, device="cuda")
+        hip.hipMemcpy(C.c_void_p(out_idx.data_ptr()), C.c_void_p(L.scn_rulebook_out_indices(rb)), n_out * 16, 3)
+        g = capi.i3()
+        L.scn_rulebook_out_grid(rb, g)
+        sets.append((out_idx, n_out, [int(v) for v in g]))
+        keep.append(rb)
+    rng = np.random.default_rng(0)
+    ch = 128
+    w = (rng.standard_normal((ch, 3, 3, 3, ch)) * 0.02).astype(np.float16)
+    b = (rng.standard_normal(ch) * 0.02).astype(np.float16)
+    ranges = np.abs(w.astype(np.float32)).reshape(ch, -1).max(1).astype(np.float32)
+    conv = L.scn_conv_create(w.ctypes.data_as(C.c_void_p), capi.i5(*w.shape), ranges.ctypes.data_as(C.c_void_p),
+                             b.ctypes.data_as(C.c_void_p), capi.PRECISION_INT8)
+    out_rows = []
+    for cur_idx, n, grid in sorted(sets, key=lambda s_: s_[1]):
+        rb = L.scn_rulebook_create(n, n, 27)
+        for _ in range(2):   # (the second build knows the row count: the launch configuration follows it)
+            capi.check(L.scn_rulebook_build_subm(rb, C.c_void_p(cur_idx.data_ptr()), n, None, capi.i3(*grid), capi.i3(3, 3, 3),
+                                                 capi.i3(1, 1, 1), st))
+            torch.cuda.synchronize()
+        offs = torch.zeros(28, dtype=torch.int64, device="cuda")
+        scratch = torch.empty(1, dtype=torch.int32, device="cuda")
+        capi.check(L.scn_rulebook_pairs(rb, C.c_void_p(scratch.data_ptr()), C.c_void_p(scratch.data_ptr()),
+                                        C.c_void_p(offs.data_ptr()), 0, st))
+        torch.cuda.synchronize()
+        pairs = int(offs.cpu().numpy()[-1])
+        x = torch.from_numpy(rng.integers(-127, 128, (n, ch)).astype(np.int8)).cuda()
+        out = torch.zeros((n, ch), dtype=torch.int8, device="cuda")
+        io = capi.ConvIO()
+        io.x_dev, io.x_ld, io.x_dynamic_range, io.relu = x.data_ptr(), ch, 3.8, 1
+        io.out_dtype, io.out_dynamic_range, io.out_dev, io.out_ld = capi.DTYPE_INT8, 6.3, out.data_ptr(), ch
+        for _ in range(5):
+            capi.check(L.scn_conv_forward(conv, rb, C.byref(io), st))
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 50
+        e0.record()
+        for _ in range(reps):
+            L.scn_conv_forward(conv, rb, C.byref(io), st)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / reps * 1e3
+        ops = 2.0 * pairs * ch * ch
+        row = {"rows": n, "grid": grid, "pairs": pairs, "pairs_per_row": round(pairs / n, 2), "us": round(us, 2),
+               "us_per_kernel_offset": round(us / 27, 3), "TOPs": round(ops / us / 1e6, 1),
+               "frac_of_int8_peak": round(ops / us / 1e6 / INT8_PEAK_TOPS, 4)}
+        out_rows.append(row)
+        print(row, file=sys.stderr, flush=True)
+        L.scn_rulebook_destroy(rb)
+    print(json.dumps({"metric": "int8 SubM 128->128 3x3x3 alone against row count (secondary figures)", "row_sweep": out_rows}))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -269,6 +409,10 @@ def main():
     t_setup = time.perf_counter()
     if args.copy_probe:
         copy_probe()
+    if args.sweep:
+        return sweep(args)
+    if args.row_sweep:
+        return row_sweep(args)
 
     # ---- workload: BASELINE.json configs[2] (int8 CenterPoint-shaped backbone, ~120k voxels)
     frame = workload.headline_points(args.points)

@@ -118,6 +118,8 @@ def build(verbose: bool = False, jobs: int = 0, incremental: bool = False) -> st
         with open(obj + ".stamp", "w") as f:
             f.write(_stamp(cmd))
 
+    if cmds and os.path.exists(LIB_PATH):
+        os.remove(LIB_PATH)    # (a build that fails must not leave the library of older sources behind)
     with ThreadPoolExecutor(max_workers=jobs_) as pool:
         list(pool.map(compile_one, cmds))
     _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-fvisibility=hidden", "-no-hip-rt", *objs, "-o", LIB_PATH],

@@ -382,7 +382,8 @@ struct Mma32<1> {
 // back from LDS.  With no staging registers the kernel fits 128 VGPRs, so two 8-wave workgroups (four
 // waves per SIMD, 512 output rows) share a CU and hide each other's latencies.
 // Hardware places lane l's bytes at base + 16 l, so the bank-conflict-free read order of the B operand is
-// obtained by permuting which chunk of its row a lane fetches: position p of a row holds chunk p ^ swz(row).
+// obtained by permuting which chunk of its row a lane fetches: position p of a row holds chunk p ^ swz(row),
+// swz(row) = (row / rows per 256 bytes) % chunks per row.
 //   iteration     = 4 K-steps = 4 KB of gathered rows per wave (32 rows x 8 chunks, or G = 8 / SEG
 //                   kernel offsets of SEG-chunk rows) and a weight slab of 4 * MT fragments
 //   LDS           = 2 weight slabs (iteration i, i+1), one 4 KB stage of gathered rows per wave, and a
@@ -411,7 +412,12 @@ __global__ __launch_bounds__(64 * WAVES, conv_lds_min_waves(CHUNKS, MT, WAVES)) 
   constexpr int SEG = CHUNKS < 8 ? CHUNKS : 8;   // chunks gathered per row and iteration
   constexpr int IPO = CHUNKS / SEG;              // iterations per kernel offset (rows wider than 128 B)
   constexpr int G = 8 / SEG;                     // kernel offsets per iteration
-  constexpr int RP = 8 / SEG;                    // rows per 128 bytes of the gathered stage
+  // Rows per rotation period of the gathered stage.  The LDS of gfx950 reads 256 bytes per clock (64 banks), so
+  // the chunk a position holds rotates over runs of 256 bytes: a stand-alone probe of ds_read_b128 of the B operand
+  // takes 1.36 times as long with the rotation over 128 bytes (the one for 32 banks) as a conflict-free read, and
+  // is level over 256.  The kernels of 128-byte rows at three workgroups per CU keep the 128-byte period: the extra
+  // shift of the longer one costs them a register they do not have (80 without scratch).
+  constexpr int RP = (CHUNKS == 8 && conv_lds_three_groups(CHUNKS, MT, WAVES) ? 8 : 16) / SEG;
   constexpr int SLAB = 4 * MT * 64;              // 16-byte weight fragments per iteration
   constexpr int NL = SLAB / 64;                  // 1 KB wave-loads per slab
   constexpr int WPT = (NL + WAVES - 1) / WAVES;  // slab loads per wave and iteration (the same for every wave:
