@@ -56,8 +56,11 @@ def parse_args():
                          "every stage of the synthetic frame, so nothing is truncated; 200000 is the exporters' figure, "
                          "at which stage 1 of that frame is cut (a secondary run)")
     ap.add_argument("--sortmask", dest="sortmask", action="store_true", default=False,
-                    help="the reference loader's sortmask switch: rows of the narrow layers' rulebooks are sorted by "
-                         "their sets of kernel offsets so that a tile visits few offsets (results are identical)")
+                    help="the reference loader's sortmask switch, a hint: the engine re-orders rows only where that is "
+                         "faster (at present nowhere, so the line equals the plain one)")
+    ap.add_argument("--tile-plans", dest="tile_plans", action="store_true", default=False,
+                    help="run every narrow layer on a tile plan sorted inside 1024-row windows, whether it pays or not "
+                         "(a measurement; results are identical)")
     ap.add_argument("--sweep", action="store_true",
                     help="latency against frame size instead of the headline line: the eight density-gradient frames of "
                          "BASELINE configuration 4 (50k - 300k points), the reference's nuScenes sweep and its 79,745-voxel "
@@ -431,7 +434,8 @@ def main():
                                     calibration_frames=[(feats.cpu().numpy(), idx.cpu().numpy())] if args.frame == "fixture" else ())
     # with_auxiliary_stream is the reference's load_engine_from_onnx option: rulebooks are built on a second
     # stream ahead of the convolutions (per-step profiling below runs them in line, on one stream)
-    eng = Engine.from_graph(graph, args.precision, with_auxiliary_stream=not args.no_aux_stream, sortmask=args.sortmask)
+    eng = Engine.from_graph(graph, args.precision, with_auxiliary_stream=not args.no_aux_stream, sortmask=args.sortmask,
+                            tile_plans=args.tile_plans)
     eng.set_input(feats, idx, GRID_ZYX)
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
@@ -533,15 +537,15 @@ def main():
     # which roof bounds the kernel: its algorithmic intensity against the machine balance (ops per HBM byte)
     intensity = dom_ops / dom_bytes
     ridge = mfma_peak * 1e12 / (HBM_PEAK_GBS * 1e9)
-    # under sortmask the narrow layers (input rows of at most 64 bytes, at most 64 output channels, kernel volume
+    # with tile plans the narrow layers (input rows of at most 64 bytes, at most 64 output channels, kernel volume
     # at most 31, all weights within 60 KB of LDS) run the tile-plan kernel
     row_bytes = -(-dom_key[0] * (1 if args.precision == "int8" else 2) // 16) * 16
     kvol, mt32 = int(np.prod(dom_key[3])), -(-dom_key[1] // 32)
-    on_plan = (args.sortmask and kvol <= 31 and mt32 <= 2 and row_bytes in (16, 32, 64)
+    on_plan = (args.tile_plans and kvol <= 31 and mt32 <= 2 and row_bytes in (16, 32, 64)
                and -(-kvol * (row_bytes // 16) // 2) * mt32 * 1024 + 512 <= 60 * 1024)
     kernel = (f"{'k_conv_tile' if on_plan else 'k_conv_lds'} {args.precision} Cin={dom_key[0]} Cout={dom_key[1]} "
               f"{'subm' if dom_key[2] else 'strided'} k={'x'.join(map(str, dom_key[3]))}")
-    traffic, traffic_from = (None, None) if args.sortmask else measured_traffic(args.precision, dom_key, nvox,
+    traffic, traffic_from = (None, None) if args.tile_plans else measured_traffic(args.precision, dom_key, nvox,
                                                                                 args.output_bound)
     # rows of every strided convolution's output: kept (what the layers after it run on) and before the
     # output_bound cut; equal unless the bound truncates
@@ -624,7 +628,7 @@ def main():
                    "active_voxels": int(nvox), "grid": list(GRID_ZYX), "output_bound": args.output_bound,
                    "truncated_by_output_bound": bool(truncated),
                    "launch": "hip graph replay" if use_graph else "direct launches",
-                   "auxiliary_stream": not args.no_aux_stream, "sortmask": bool(args.sortmask), "output": out_view.shape},
+                   "auxiliary_stream": not args.no_aux_stream, "sortmask": bool(args.sortmask), "tile_plans": bool(args.tile_plans), "output": out_view.shape},
         "voxels_per_s": round(nvox * 1e3 / ms_per_step, 1),
         "voxelization_ms": round(vox_ms, 4),
         "host_enqueue_ms_per_step": round(enqueue_ms, 4),

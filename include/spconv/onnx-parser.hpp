@@ -15,7 +15,9 @@ namespace spconv {
  * onnx_file: the custom "scn" ONNX dialect written by the reference's exporters.
  * precision: Float16 forces every layer to fp16; Int8 honours the per-layer precision attributes
  *            (layers without dynamic ranges stay fp16).
- * sortmask / enable_blackwell / with_auxiliary_stream: accepted for source compatibility, ignored.
+ * sortmask: a hint, passed on (the engine re-orders rows only where that is faster; results never change).
+ * with_auxiliary_stream: passed on (rulebooks are built on a second stream ahead of the convolutions).
+ * enable_blackwell: accepted for source compatibility, ignored.
  * stream: the stream used for one-time uploads; avoid the default stream for forward().
  */
 inline std::shared_ptr<Engine> load_engine_from_onnx(const std::string& onnx_file, Precision precision = Precision::Float16,

@@ -15,7 +15,7 @@ OK = 0
 PRECISION_FP16, PRECISION_INT8 = 1, 2
 DTYPE_INT32, DTYPE_FP16, DTYPE_FP32, DTYPE_INT8 = 1, 2, 3, 7
 ORDER_XYZ, ORDER_ZYX = 1, 2
-BUILD_SORTMASK, BUILD_AUX_STREAM, BUILD_KEEP_ALL = 1, 4, 256
+BUILD_SORTMASK, BUILD_AUX_STREAM, BUILD_KEEP_ALL, BUILD_TILE_PLANS = 1, 4, 256, 512
 
 vp = C.c_void_p
 u32 = C.c_uint32

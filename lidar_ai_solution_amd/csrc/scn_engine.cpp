@@ -173,7 +173,7 @@ struct RbSlot {
   int inverse_of = -1;   // >= 0: the strided rulebook this one swaps (SparseInverseConvolution)
   bool initialised = false;
   bool want_plan = false;   // some convolution on this rulebook runs the tile-plan kernel
-  bool plan_sorted = false; // ... with the rows sorted by their offset sets (SCN_BUILD_SORTMASK)
+  bool plan_sorted = false; // ... with the rows sorted by their offset sets (SCN_BUILD_TILE_PLANS)
 };
 
 }  // namespace scn
@@ -475,10 +475,14 @@ static bool build_engine(scn_engine& e) {
                      n.bias.empty() ? nullptr : n.bias.data(), comp))
           return false;
         const int ci = (int)e.convs.size();
-        // sortmask: the narrow layers run on sorted tile plans.  (Without the switch no plan is built: in row
-        // order the tile-plan kernel is level with the LDS-staged one, and the masks would cost the first
-        // rulebook of a frame 9 us on the critical path.)
-        if ((e.flags & SCN_BUILD_SORTMASK) && slot.inverse_of < 0 && conv_tile_covers(*w)) {
+        // Tile plans: the narrow layers run the tile-plan kernel on rows sorted by offset set inside 1024-row windows.
+        // Built only on request (SCN_BUILD_TILE_PLANS).  The reference's sortmask flag is a hint to skip more empty
+        // work where that is faster, and on this GPU it is faster nowhere: measured on a 123,646-voxel frame, plans
+        // cost the first four rulebooks 30 .. 60 us each (masks, sort, re-ordered table), the 16-channel layers stay
+        // within 2 us and the 32-channel layers go from 27 to 37 .. 45 us (re-ordered rows gather with less
+        // locality); in row order (masks only) the tile-plan kernel is level with the LDS-staged one and the masks
+        // still cost 10 us per rulebook.  So SCN_BUILD_SORTMASK alone builds no plan.
+        if ((e.flags & SCN_BUILD_TILE_PLANS) && slot.inverse_of < 0 && conv_tile_covers(*w)) {
           slot.want_plan = true;
           slot.plan_sorted = true;
         }

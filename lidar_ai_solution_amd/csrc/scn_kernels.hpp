@@ -64,12 +64,11 @@ struct ConvGeom {
 // Tile plan of a rulebook: what lets a convolution skip the kernel offsets at which none of a 32-row tile's rows
 // has a neighbour (`sortmask` of the reference's loader, libraries/3DSparseConvolution/src/onnx-parser.hpp:35-37:
 // "skip more insignificance computations").  tmask[t] = OR of the rows' offset sets (bit k: nbr[k][row] >= 0).
-// A sorted plan also orders the rows by their offset set (stable radix sort of the sets as numbers), so that the
-// rows of a tile share most offsets: perm[j] = row at position j, nbr = the table in that order.  Results do not
+// A sorted plan also orders the rows by their offset set (stable, the sets as numbers, inside windows of 1024
+// consecutive rows), so that the rows of a tile share most offsets: perm[j] = row at position j, nbr = the table in that order.  Results do not
 // depend on the plan: every row still adds its own products in offset order.
 struct TilePlan {
-  DevBuf keys, keys_sorted, rows, perm, tmask, nbr, temp;
-  size_t temp_bytes = 0;
+  DevBuf keys, keys_sorted, perm, tmask, nbr;
   uint32_t cap_rows = 0;   // positions allocated (multiple of 32)
   bool reserved_sorted = false;
   bool sorted = false;     // what the last build produced

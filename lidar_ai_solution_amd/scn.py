@@ -97,16 +97,18 @@ class Engine:
     @classmethod
     def from_onnx(cls, path: str, precision="fp16", sortmask=False, enable_blackwell=False, with_auxiliary_stream=False,
                   fixed_launch_points: int = 10000, stream=None, keep_all: bool = False,
-                  precision_overrides=(), tensor_ranges=None) -> "Engine":
+                  precision_overrides=(), tensor_ranges=None, tile_plans: bool = False) -> "Engine":
         """spconv::load_engine_from_onnx.  Raises instead of returning nullptr on failure.
 
         precision_overrides: (selector, by_optype, precision, output_precision) tuples applied to the
         nodes' precisions before the engine is planned -- the older interface's set_node_precision_byname /
         set_node_precision_byoptype + reconfigure; precision None leaves the model's value.
         tensor_ranges: {tensor name: calibrated |max|} (see collect_amax); replaces the dynamic ranges of the
-        model's convolutions and Adds."""
+        model's convolutions and Adds.
+        sortmask is the reference's hint (the engine re-orders rows only where that is faster: at present nowhere);
+        tile_plans runs every narrow layer on a sorted tile plan regardless."""
         flags = (capi.BUILD_SORTMASK if sortmask else 0) | (capi.BUILD_AUX_STREAM if with_auxiliary_stream else 0) | \
-                (capi.BUILD_KEEP_ALL if keep_all else 0)
+                (capi.BUILD_KEEP_ALL if keep_all else 0) | (capi.BUILD_TILE_PLANS if tile_plans else 0)
         n = len(precision_overrides)
         arr = (capi.PrecisionOverride * max(n, 1))()
         for i, (sel, by_optype, prec, out_prec) in enumerate(precision_overrides):
@@ -127,7 +129,7 @@ class Engine:
 
     @classmethod
     def from_graph(cls, graph: Graph, precision="fp16", keep_all: bool = False,
-                   with_auxiliary_stream: bool = False, sortmask: bool = False) -> "Engine":
+                   with_auxiliary_stream: bool = False, sortmask: bool = False, tile_plans: bool = False) -> "Engine":
         """Drives the EngineBuilder calls (push_input / push_sparse_conv / ... / build) node by node,
         the way `onnx-parser.cpp:116-230` does."""
         L = capi.lib()
@@ -177,7 +179,7 @@ class Engine:
             for name in graph.outputs:
                 capi.check(L.scn_builder_push_output(b, tmap[name]))
             flags = (capi.BUILD_KEEP_ALL if keep_all else 0) | (capi.BUILD_AUX_STREAM if with_auxiliary_stream else 0) | \
-                    (capi.BUILD_SORTMASK if sortmask else 0)
+                    (capi.BUILD_SORTMASK if sortmask else 0) | (capi.BUILD_TILE_PLANS if tile_plans else 0)
             h = L.scn_builder_build(b, _prec(precision), flags, None)
         finally:
             L.scn_builder_destroy(b)

@@ -750,8 +750,8 @@ def test_launch_configuration_chosen_for_a_small_frame_serves_a_large_one(cp_mod
     f, i = to_dev(feats), to_dev(idx)
     cnt = torch.tensor([3000], dtype=torch.int32, device=DEV)
     for aux in (False, True):
-        note(f"small frame, then the full one on launches chosen for the small one (auxiliary stream / sortmask {aux})")
-        eng = Engine.from_graph(g8, "int8", with_auxiliary_stream=aux, sortmask=aux)
+        note(f"small frame, then the full one on launches chosen for the small one (auxiliary stream / tile plans {aux})")
+        eng = Engine.from_graph(g8, "int8", with_auxiliary_stream=aux, sortmask=aux, tile_plans=aux)
         eng.set_input(f, i, GRID_ZYX)
         eng.set_dds_num_of_points_pointer(cnt)
         cnt.fill_(3000)
@@ -903,7 +903,7 @@ def test_graph_with_three_outputs_dense_and_intermediate_sparse(rows, centerpoin
                        ("fused, auxiliary stream", lambda: Engine.from_graph(g8, "int8", with_auxiliary_stream=True)),
                        ("every tensor kept", lambda: Engine.from_graph(g8, "int8", keep_all=True)),
                        ("loaded from the model file", lambda: Engine.from_onnx(path, "int8")),
-                       ("sortmask", lambda: Engine.from_graph(g8, "int8", sortmask=True))):
+                       ("tile plans", lambda: Engine.from_graph(g8, "int8", sortmask=True, tile_plans=True))):
         note(f"three-output int8 graph on {rows} rows: {what}")
         eng = make()
         _run_engine(eng, feats, idx, GRID_ZYX)

@@ -1,5 +1,5 @@
 """Tile plans (the reference loader's `sortmask` switch) and the tile-plan convolution kernel of the narrow
-layers: the plan is what its definition says (masks, a permutation sorted by offset set, the table in plan
+layers: the plan is what its definition says (masks, a permutation sorted by offset set inside 1024-row windows, the table in plan
 order), and convolutions with a plan -- in row order and sorted -- give the bits of the plan-less kernels and of
 the CPU oracle.  Needs a MI355X."""
 import ctypes as C
@@ -69,7 +69,9 @@ def test_plan_is_what_it_says(kind, centerpoint_input):
     note(f"sorted tile plan, {kind} rulebook")
     capi.check(L.scn_rulebook_build_plan(rb.h, 1, stream()))
     tmask, perm, tab = _plan_of(rb, n, 27)
-    order = np.argsort(masks, kind="stable")                      # the definition: stable sort by offset set
+    # the definition: stable sort by offset set inside windows of 1024 consecutive rows
+    order = np.concatenate([b + np.argsort(masks[b:b + 1024], kind="stable") for b in range(0, n, 1024)])
+    assert np.all(order // 1024 == np.arange(n) // 1024)
     assert np.array_equal(perm[:n], order.astype(np.uint32))
     assert np.all(perm[n:] >= n)
     sorted_masks = np.zeros(pos, np.uint32)
@@ -227,7 +229,8 @@ def test_plan_with_device_side_count_and_empty_input():
 
 
 def test_engine_sortmask_gives_identical_results(centerpoint_input, bevfusion_input):
-    """`sortmask` of load_engine_from_onnx / EngineBuilder::build: the narrow layers run on sorted tile plans.
+    """Engines built with tile plans (`sortmask` of load_engine_from_onnx / EngineBuilder::build is the hint; the
+    plans themselves are switched on by SCN_BUILD_TILE_PLANS): the narrow layers run on sorted tile plans.
     Every kept tensor of the int8 CenterPoint-shaped engine and the BEV outputs of the fused int8 / fp16 engines,
     with and without an auxiliary stream, equal the plain engine's bit for bit; a second, smaller frame on the
     same engines too (no stale plan)."""
@@ -241,7 +244,7 @@ def test_engine_sortmask_gives_identical_results(centerpoint_input, bevfusion_in
     graphs.apply_int8_plan(g8, tags8, amax, "centerpoint")
     note("int8 engine, every tensor kept: sortmask vs plain")
     plain = Engine.from_graph(g8, "int8", keep_all=True)
-    sort = Engine.from_graph(g8, "int8", keep_all=True, sortmask=True)
+    sort = Engine.from_graph(g8, "int8", keep_all=True, sortmask=True, tile_plans=True)
     _run_engine(plain, feats, idx, GRID_ZYX)
     _run_engine(sort, feats, idx, GRID_ZYX)
     checked = 0
@@ -259,7 +262,7 @@ def test_engine_sortmask_gives_identical_results(centerpoint_input, bevfusion_in
         want_eng = Engine.from_graph(graph, prec)
         for aux in (False, True):
             note(f"fused {prec} engine with sortmask, auxiliary stream {aux}: two frames")
-            eng = Engine.from_graph(graph, prec, sortmask=True, with_auxiliary_stream=aux)
+            eng = Engine.from_graph(graph, prec, sortmask=True, tile_plans=True, with_auxiliary_stream=aux)
             for rows in (feats.shape[0], 23456, feats.shape[0]):
                 _run_engine(want_eng, feats[:rows], idx[:rows], GRID_ZYX)
                 want = want_eng.output(0).torch().clone()
@@ -272,7 +275,7 @@ def test_engine_sortmask_gives_identical_results(centerpoint_input, bevfusion_in
     bamax = _oracle_calibration(b16, bf, bi, GRID_XYZ)
     b8, bt8 = graphs.bevfusion_scn(seed=1)
     graphs.apply_int8_plan(b8, bt8, bamax, "bevfusion")
-    e0, e1 = Engine.from_graph(b8, "int8"), Engine.from_graph(b8, "int8", sortmask=True)
+    e0, e1 = Engine.from_graph(b8, "int8"), Engine.from_graph(b8, "int8", sortmask=True, tile_plans=True)
     _run_engine(e0, bf, bi, GRID_XYZ)
     _run_engine(e1, bf, bi, GRID_XYZ)
     assert torch.equal(e0.output(0).torch().view(torch.int16), e1.output(0).torch().view(torch.int16))
