@@ -918,11 +918,29 @@ struct VoxGeom {
   int max_voxels, max_pts;
 };
 
+// The voxelizer keeps its working memory clean between calls instead of clearing it at the start of each:
+//   cells     uint2 per 32 cells: .x occupancy bits, .y rank of the word's first bit.  Bits are cleared at the end of
+//             the forward that set them, one store per point (k_vox_mean).
+//   flags     one word per block of 1024 words: some cell of the block is occupied; cleared the same way.  (Walking
+//             a second-level bitmap of the occupied words instead -- one thread per 32 words, 82 workgroups -- was
+//             measured at 16 + 46 us for the two rank passes against 5 + 17 us: few threads with dependent loads.)
+//   slots     [max_voxels][max_points] point indices tagged in the top 8 bits.  A forward uses two tags, 2e + 1 for
+//             the slots filled in arrival order and 2e for the cascade of the voxels that overflow, and e counts
+//             DOWN: every value of an earlier call (or phase) is larger than any value of the current one, so to the
+//             atomicMin cascade a stale slot is an empty one.  (A full clear every 127 calls, when the tags wrap.)
+// Atomics that every XCD must see are the cost of this stage (they are served by the memory side, not by an XCD's L2),
+// so a point costs two: the occupancy bit, and its voxel's counter, whose old value is its slot.  A voxel that
+// receives more than max_points points needs the lowest indices among them, which arrival order does not give: those
+// voxels' points (none in most frames: the pass leaves at once when no counter overflowed) go through a cascade.
+// One forward = mark, block sums, rank, assign, overflow, mean.
+constexpr uint32_t kVoxTagShift = 24;     // point indices stay below 2^24
+constexpr uint32_t kVoxEpochs = 127;      // epochs 126 .. 0 (tags 253 .. 0); 255 is what a cleared slot holds
+
 // Pass 1 over the point stream (PT: fp16 points, or the fp32 points of CUDA-CenterPoint's preprocessing,
-// src/preprocess_kernels.cu:70-98): cell key per point + occupancy bit.
+// src/preprocess_kernels.cu:70-98): cell key per point, occupancy bit, and the flag of the cell's block.
 template <typename PT>
 __global__ __launch_bounds__(256) void k_vox_mark(const PT* __restrict__ pts, uint32_t n, VoxGeom g,
-                                                  uint32_t* pkey, uint32_t* bitmap) {
+                                                  uint32_t* pkey, uint2* cells, uint32_t* flags) {
   const uint32_t p = blockIdx.x * 256 + threadIdx.x;
   if (p >= n) return;
   const float px = (float)pts[(size_t)p * g.nf + 0];
@@ -936,56 +954,275 @@ __global__ __launch_bounds__(256) void k_vox_mark(const PT* __restrict__ pts, ui
     if (ix >= 0 && ix < g.g[0] && iy >= 0 && iy < g.g[1] && iz >= 0 && iz < g.g[2]) {
       key = g.order == SCN_ORDER_ZYX ? ((uint32_t)iz * g.g[1] + iy) * g.g[0] + ix
                                      : ((uint32_t)ix * g.g[1] + iy) * g.g[2] + iz;
-      atomicOr(&bitmap[key >> 5], 1u << (key & 31));
+      const uint32_t bit = 1u << (key & 31);
+      const uint32_t old = atomicOr(&cells[key >> 5].x, bit);
+      if (!(old & bit)) flags[key >> 15] = 1u;   // (1024 words of 32 cells per block)
     }
   }
   pkey[p] = key;
 }
 
-// Pass 2: voxel id = rank of the cell; count the point and keep the max_pts lowest point indices
-// of the voxel, sorted, with an atomicMin cascade (slot j ends up holding the j-th smallest index
-// whatever the arrival order).
-__global__ __launch_bounds__(256) void k_vox_assign(const uint32_t* __restrict__ pkey, uint32_t n,
-                                                    const uint32_t* __restrict__ bitmap,
-                                                    const uint32_t* __restrict__ prefix, int max_voxels, int max_pts,
-                                                    uint32_t* counts, uint32_t* mins) {
-  const uint32_t p = blockIdx.x * 256 + threadIdx.x;
-  if (p >= n) return;
-  const uint32_t key = pkey[p];
-  if (key == 0xFFFFFFFFu) return;
-  const uint32_t w = key >> 5, b = key & 31;
-  const uint32_t id = prefix[w] + __popc(bitmap[w] & ((1u << b) - 1u));
-  if (id >= (uint32_t)max_voxels) return;
-  atomicAdd(&counts[id], 1u);
-  uint32_t x = p;
-  uint32_t* slot = mins + (size_t)id * max_pts;
-  for (int j = 0; j < max_pts; ++j) {
-    const uint32_t old = atomicMin(&slot[j], x);
-    if (old == 0xFFFFFFFFu) break;  // slot was empty: nothing is displaced
-    x = old > x ? old : x;
+// Pass 2a: occupied cells per block of 1024 words; a block whose flag is down is not read.
+__global__ __launch_bounds__(256) void k_vox_blocksum(const uint2* __restrict__ cells, const uint32_t* __restrict__ flags,
+                                                      uint32_t* blocksum) {
+  __shared__ uint32_t scratch[17];
+  if (flags[blockIdx.x] == 0) {   // (the whole workgroup)
+    if (threadIdx.x == 0) blocksum[blockIdx.x] = 0;
+    return;
+  }
+  const uint4* w = reinterpret_cast<const uint4*>(cells + (size_t)blockIdx.x * 1024);   // two words' (bits, rank) each
+  uint32_t c = 0;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const uint4 v = w[j * 256 + threadIdx.x];
+    c += __popc(v.x) + __popc(v.z);
+  }
+  uint32_t total;
+  (void)block_exclusive_scan(c, scratch, &total);
+  if (threadIdx.x == 0) blocksum[blockIdx.x] = total;
+}
+
+// Pass 2b, one workgroup per block of 1024 words (four per thread): ranks.  Every block with an occupied cell adds up
+// the counts of the blocks before it, writes the rank of each occupied word's first bit next to its bits and the
+// coordinate rows of its cells; the last block publishes the totals; all of them zero the per-voxel point counts.
+__global__ __launch_bounds__(256) void k_vox_rank(uint2* cells, const uint32_t* __restrict__ blocksum, Int3 grid,
+                                                  uint32_t cap, int4* coords_out, uint32_t* counters,
+                                                  uint32_t* counts) {
+  __shared__ uint32_t scratch[17];
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < cap; i += (size_t)gridDim.x * 256) counts[i] = 0;
+  const uint32_t own = blocksum[blockIdx.x];
+  if (own == 0 && blockIdx.x != gridDim.x - 1) return;   // (the whole workgroup; the last block publishes the totals)
+  uint32_t part = 0;
+  for (uint32_t i = threadIdx.x; i < blockIdx.x; i += 256) part += blocksum[i];
+  uint32_t base;
+  (void)block_exclusive_scan(part, scratch, &base);
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+    const uint32_t all = base + own;
+    counters[1] = all;
+    counters[0] = all < cap ? all : cap;
+  }
+  if (own == 0) return;   // (the whole workgroup)
+  const size_t w0 = (size_t)blockIdx.x * 1024 + (size_t)threadIdx.x * 4;
+  uint32_t bits[4];
+  uint32_t c = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    bits[j] = cells[w0 + j].x;
+    c += __popc(bits[j]);
+  }
+  uint32_t total;
+  uint32_t rank = base + block_exclusive_scan(c, scratch, &total);
+  if (c == 0) return;
+  const uint32_t g12 = (uint32_t)grid.v[1] * (uint32_t)grid.v[2];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    uint32_t bj = bits[j];
+    if (bj == 0) continue;
+    cells[w0 + j].y = rank;
+    while (bj) {
+      const int b = __ffs(bj) - 1;
+      bj &= bj - 1;
+      if (rank < cap) {
+        const uint32_t key = (uint32_t)(w0 + j) * 32u + (uint32_t)b;
+        const uint32_t i0 = key / g12, rem = key - i0 * g12;
+        const uint32_t i1 = rem / (uint32_t)grid.v[2], i2 = rem - i1 * (uint32_t)grid.v[2];
+        coords_out[rank] = make_int4(0, (int)i0, (int)i1, (int)i2);
+      }
+      rank++;
+    }
   }
 }
 
-// Pass 3: per voxel mean of the kept points, summed in point-index order in fp32.
+// Lanes of a wave that follow each other with the same cell (a real sweep lists its points ring by ring): the run's
+// first lane, its length, and this lane's place in it.  All 64 lanes call this.
+struct VoxRun {
+  int start, len, pos;
+};
+__device__ __forceinline__ VoxRun vox_run(uint32_t key, int lane) {
+  const uint32_t prev = (uint32_t)__shfl_up((int)key, 1, 64);
+  const bool head = lane == 0 || key != prev;
+  const uint64_t heads = __ballot(head);
+  const uint64_t upto = heads & (lane == 63 ? ~0ull : ((2ull << lane) - 1ull));   // heads at or below this lane
+  const int start = 63 - __clzll((long long)upto);
+  const uint64_t above = lane == 63 ? 0ull : heads & ~((2ull << lane) - 1ull);
+  const int end = above ? __ffsll((long long)above) - 1 : 64;
+  VoxRun r;
+  r.start = start;
+  r.len = end - start;
+  r.pos = lane - start;
+  return r;
+}
+
+// Pass 3: voxel id = rank of the cell; the voxel's counter gives the point its slot (arrival order; a run of lanes
+// with one cell adds its length once and takes consecutive slots).  Raises *overflow when a voxel receives more
+// points than it has slots.
+__global__ __launch_bounds__(256) void k_vox_assign(const uint32_t* __restrict__ pkey, uint32_t n,
+                                                    const uint2* __restrict__ cells, int max_voxels, int max_pts,
+                                                    uint32_t tag, uint32_t* counts, uint32_t* slots, uint32_t* overflow,
+                                                    int always) {
+  const uint32_t p = blockIdx.x * 256 + threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  if (always && p == 0) *overflow = 1u;   // (more slots than pass 4 puts in order: every voxel goes through pass 3b)
+  const uint32_t key = p < n ? pkey[p] : 0xFFFFFFFFu;
+  const VoxRun r = vox_run(key, lane);
+  uint32_t id = 0xFFFFFFFFu;
+  if (key != 0xFFFFFFFFu) {
+    const uint2 ci = cells[key >> 5];
+    id = ci.y + __popc(ci.x & ((1u << (key & 31)) - 1u));
+  }
+  const bool take = id < (uint32_t)max_voxels;
+  uint32_t base = 0;
+  if (take && r.pos == 0) base = atomicAdd(&counts[id], (uint32_t)r.len);
+  base = (uint32_t)__shfl((int)base, r.start, 64);
+  if (!take) return;
+  const uint32_t at = base + (uint32_t)r.pos;
+  if (at < (uint32_t)max_pts)
+    slots[(size_t)id * max_pts + at] = (tag << kVoxTagShift) | p;
+  else if (at == (uint32_t)max_pts)
+    *overflow = 1u;
+}
+
+// Pass 3b, only for frames in which some voxel overflowed: every point of such a voxel enters an atomicMin cascade
+// over the voxel's slots (slot j ends up holding the j-th smallest index whatever the arrival order; the slots that
+// pass 3 filled carry the larger tag and count as empty).  Of a run of lanes only the first max_pts can be among the
+// max_pts lowest.  Two launches: the first lanes of the runs (phase 0), then the others (phase 1).  A voxel next to
+// the sensor holds a thousand points in a hundred runs, and read-modify-writes on one 64-byte line are carried out one
+// after the other by the memory side, about ten per microsecond: all candidates at once are over a thousand of them
+// (135 us on the reference's demo sweep), while after phase 0 the slots hold ten low indices and nearly every
+// other candidate leaves on the reads in front of the cascade.
+__global__ __launch_bounds__(256) void k_vox_overflow(const uint32_t* __restrict__ pkey, uint32_t n,
+                                                      const uint2* __restrict__ cells, int max_voxels, int max_pts,
+                                                      uint32_t tag, const uint32_t* __restrict__ counts, uint32_t* slots,
+                                                      const uint32_t* __restrict__ overflow, int always, int phase) {
+  if (*overflow == 0) return;
+  const int lane = threadIdx.x & 63;
+  // (whole waves run every round of the loop: the run bookkeeping is wave-wide)
+  for (uint32_t p0 = blockIdx.x * 256; p0 < n; p0 += gridDim.x * 256) {
+    const uint32_t p = p0 + threadIdx.x;
+    const uint32_t key = p < n ? pkey[p] : 0xFFFFFFFFu;
+    const VoxRun r = vox_run(key, lane);
+    if (key == 0xFFFFFFFFu || r.pos >= max_pts || (phase == 0) != (r.pos == 0)) continue;
+    const uint2 ci = cells[key >> 5];
+    const uint32_t id = ci.y + __popc(ci.x & ((1u << (key & 31)) - 1u));
+    if (id >= (uint32_t)max_voxels || (!always && counts[id] <= (uint32_t)max_pts)) continue;
+    uint32_t x = (tag << kVoxTagShift) | p;
+    uint32_t* slot = slots + (size_t)id * max_pts;
+    // A voxel of hundreds of points (next to the sensor) would send every one of them down the same ten addresses,
+    // starting with the first.  Slot values only fall and stay in ascending order, so the slots that hold less than
+    // this point now (plain loads) will always do: the point enters the cascade behind them, and not at all when
+    // that is every slot.
+    // (Loads at device scope: the atomics are carried out by the memory side, and an ordinary load could be served
+    // from a copy that never sees them.  Read-modify-writes on one 64-byte line run one after the other, at about ten
+    // per microsecond: without these reads the frame's fullest voxel alone sets the time of the pass.)
+    const uint32_t last = __hip_atomic_load(&slot[max_pts - 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((last >> kVoxTagShift) == tag && last < x) continue;
+    int j0 = 0;
+    for (; j0 < max_pts; ++j0) {
+      const uint32_t cur = __hip_atomic_load(&slot[j0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if ((cur >> kVoxTagShift) != tag || cur > x) break;
+    }
+    for (int j = j0; j < max_pts; ++j) {
+      const uint32_t old = atomicMin(&slot[j], x);
+      if ((old >> kVoxTagShift) != tag) break;  // the slot was empty (cleared, an earlier call's, or pass 3's): nothing is displaced
+      x = old > x ? old : x;
+    }
+  }
+}
+
+// Mean of cnt <= N points whose indices stand in slot[] in any order: indices through a bitonic network (ascending,
+// padding last), values added in that order in fp32.  N a power of two; nf <= kVoxMaxFeatures.
+constexpr int kVoxMaxSlots = 16;
+constexpr int kVoxMaxFeatures = 8;
+template <typename PT, int N>
+__device__ __forceinline__ void vox_ordered_mean(const PT* __restrict__ pts, const uint32_t* __restrict__ slot, uint32_t cnt,
+                                                 int nf, _Float16* out) {
+  const uint32_t pmask = (1u << kVoxTagShift) - 1u;
+  uint32_t idx[N];
+#pragma unroll
+  for (int j = 0; j < N; ++j) idx[j] = (uint32_t)j < cnt ? slot[j] & pmask : 0xFFFFFFFFu;
+#pragma unroll
+  for (int k = 2; k <= N; k <<= 1)
+#pragma unroll
+    for (int d = k >> 1; d > 0; d >>= 1)
+#pragma unroll
+      for (int i = 0; i < N; ++i) {
+        const int l = i ^ d;
+        if (l > i) {
+          const bool up = (i & k) == 0;
+          const uint32_t a = idx[i], b = idx[l];
+          const bool sw = (a > b) == up;
+          idx[i] = sw ? b : a;
+          idx[l] = sw ? a : b;
+        }
+      }
+  float s[kVoxMaxFeatures];
+#pragma unroll
+  for (int f = 0; f < kVoxMaxFeatures; ++f) s[f] = 0.f;
+#pragma unroll
+  for (int r = 0; r < N; ++r) {
+    if ((uint32_t)r < cnt) {
+      const PT* q = pts + (size_t)idx[r] * nf;
+#pragma unroll
+      for (int f = 0; f < kVoxMaxFeatures; ++f)
+        if (f < nf) {
+          const float x = (float)q[f];
+          s[f] = r == 0 ? x : s[f] + x;
+        }
+    }
+  }
+#pragma unroll
+  for (int f = 0; f < kVoxMaxFeatures; ++f)
+    if (f < nf) out[f] = (_Float16)(s[f] / (float)cnt);
+}
+
+// Pass 4, one thread per voxel: mean of the kept points, summed in point-index order in fp32 (slots in arrival order
+// are put in order first, by a sorting network over at most 16 of them); and, one thread per point, the occupancy bits
+// and block flags of this frame back to zero for the next one.
 template <typename PT>
 __global__ __launch_bounds__(256) void k_vox_mean(const PT* __restrict__ pts, const uint32_t* n_vox_dev,
                                                   int max_voxels, int max_pts, int nf,
                                                   const uint32_t* __restrict__ counts,
-                                                  const uint32_t* __restrict__ mins, _Float16* feats) {
-  const uint32_t nv = eff_n(n_vox_dev, (uint32_t)max_voxels);
+                                                  const uint32_t* __restrict__ slots, _Float16* feats,
+                                                  const uint32_t* __restrict__ pkey, uint32_t n_points, uint2* cells,
+                                                  uint32_t* flags, uint32_t* overflow) {
   const uint32_t t = blockIdx.x * 256 + threadIdx.x;
-  const uint32_t v = t / nf, f = t % nf;
-  if (v >= nv) return;
-  uint32_t cnt = counts[v];
-  if (cnt > (uint32_t)max_pts) cnt = max_pts;
-  const uint32_t* slot = mins + (size_t)v * max_pts;
-  float s = 0.f;
-  for (uint32_t j = 0; j < cnt; ++j) {
-    const float x = (float)pts[(size_t)slot[j] * nf + f];
-    s = j == 0 ? x : s + x;
+  if (t == 0) *overflow = 0;   // (pass 3b of this forward has run)
+  if (t < n_points) {
+    const uint32_t key = pkey[t];
+    if (key != 0xFFFFFFFFu) {
+      cells[key >> 5].x = 0;
+      flags[key >> 15] = 0;
+    }
   }
-  s = s / (float)cnt;
-  feats[(size_t)v * nf + f] = (_Float16)s;
+  const uint32_t nv = eff_n(n_vox_dev, (uint32_t)max_voxels);
+  const uint32_t v = t;
+  if (v >= nv) return;
+  const uint32_t all = counts[v];
+  const uint32_t cnt = all > (uint32_t)max_pts ? (uint32_t)max_pts : all;
+  const uint32_t* slot = slots + (size_t)v * max_pts;
+  const uint32_t pmask = (1u << kVoxTagShift) - 1u;
+  _Float16* out = feats + (size_t)v * nf;
+  if (all > (uint32_t)max_pts || max_pts > kVoxMaxSlots || nf > kVoxMaxFeatures) {
+    // in order already (the cascade's result: see the host side for max_pts > 16), or more features than the
+    // registers below hold
+    for (int f = 0; f < nf; ++f) {
+      float s = 0.f;
+      for (uint32_t j = 0; j < cnt; ++j) {
+        const float x = (float)pts[(size_t)(slot[j] & pmask) * nf + f];
+        s = j == 0 ? x : s + x;
+      }
+      out[f] = (_Float16)(s / (float)cnt);
+    }
+    return;
+  }
+  if (cnt <= 2)
+    vox_ordered_mean<PT, 2>(pts, slot, cnt, nf, out);
+  else if (cnt <= 4)
+    vox_ordered_mean<PT, 4>(pts, slot, cnt, nf, out);
+  else if (cnt <= 8)
+    vox_ordered_mean<PT, 8>(pts, slot, cnt, nf, out);
+  else
+    vox_ordered_mean<PT, kVoxMaxSlots>(pts, slot, cnt, nf, out);
 }
 
 }  // namespace scn
@@ -1058,11 +1295,23 @@ scn_voxelizer* scn_voxelizer_create(const scn_voxelization_param* param) {
   v->p = *param;
   v->words = bitmap_words_for(g);
   const size_t mv = (size_t)param->max_voxels;
-  bool ok = v->bitmap.alloc(v->words * 4) && v->prefix.alloc(v->words * 4) &&
-            v->blocksum.alloc((v->words / kWordsPerBlock + 1) * 4) && v->pkey.alloc((size_t)param->max_points * 4) &&
+  if ((uint64_t)param->max_points >= (1ull << kVoxTagShift)) {
+    set_error("scn_voxelizer_create: max_points must be below 2^24");
+    delete v;
+    return nullptr;
+  }
+  // bitmap: uint2 per word (bits, rank of the first bit); clean = zero bits, zero block counts, cleared slots
+  bool ok = v->bitmap.alloc(v->words * 8) && v->blocksum.alloc((v->words / kWordsPerBlock + 1) * 4) &&
+            v->flags.alloc((v->words / kWordsPerBlock + 1) * 4) &&
+            v->pkey.alloc((size_t)param->max_points * 4) &&
             v->mins.alloc(mv * param->max_points_per_voxel * 4) && v->counts.alloc(mv * 4) &&
             v->feats.alloc(mv * param->num_feature * 2) && v->idx.alloc(mv * 16) && v->counters.alloc(64);
-  if (ok) ok = hipMemset(v->counters.p, 0, 64) == hipSuccess && hipMemset(v->idx.p, 0, mv * 16) == hipSuccess &&
+  if (ok) ok = hipMemset(v->bitmap.p, 0, v->words * 8) == hipSuccess &&
+               hipMemset(v->blocksum.p, 0, (v->words / kWordsPerBlock + 1) * 4) == hipSuccess &&
+               hipMemset(v->flags.p, 0, (v->words / kWordsPerBlock + 1) * 4) == hipSuccess &&
+               hipMemset(v->mins.p, 0xFF, mv * param->max_points_per_voxel * 4) == hipSuccess &&
+               hipMemset(v->counts.p, 0, mv * 4) == hipSuccess &&
+               hipMemset(v->counters.p, 0, 64) == hipSuccess && hipMemset(v->idx.p, 0, mv * 16) == hipSuccess &&
                hipMemset(v->feats.p, 0, mv * param->num_feature * 2) == hipSuccess &&
                hipHostMalloc((void**)&v->host_count, sizeof(uint32_t), hipHostMallocDefault) == hipSuccess;
   if (!ok) {
@@ -1115,40 +1364,50 @@ int scn_voxelizer_forward_points(scn_voxelizer* v, const void* points_fp16_dev, 
   g.max_voxels = p.max_voxels;
   g.max_pts = p.max_points_per_voxel;
   v->last_order = order;
-  // one launch clears the cell bitmap, the per-voxel point slots and the per-voxel counts
-  const FillJob clears[3] = {{v->bitmap.p, v->words, 0u},
-                             {v->mins.p, (size_t)p.max_voxels * p.max_points_per_voxel, 0xFFFFFFFFu},
-                             {v->counts.p, (size_t)p.max_voxels, 0u}};
-  int rc = fill_multi(clears, 3, nullptr, nullptr, 0, stream);
-  if (rc) return rc;
+  // (the working memory is clean: see the kernels.  The slots' tags count down; when they are used up the slots are cleared.)
+  if (v->epoch == 0) {
+    int rc = fill_u32(v->mins.p, 0xFFFFFFFFu, (size_t)p.max_voxels * p.max_points_per_voxel, stream);
+    if (rc) return rc;
+    v->epoch = kVoxEpochs;
+  }
+  const uint32_t epoch = --v->epoch;
+  const uint32_t tag_arrival = 2 * epoch + 1, tag_cascade = 2 * epoch;
+  // (more slots or features than pass 4 puts in order in registers: every voxel goes through the cascade of pass 3b)
+  const int always = (p.max_points_per_voxel > kVoxMaxSlots || p.num_feature > kVoxMaxFeatures) ? 1 : 0;
   uint32_t* cnt = v->counters.as<uint32_t>();
+  uint32_t* overflow = cnt + 4;
+  uint2* cells = reinterpret_cast<uint2*>(v->bitmap.p);
+  uint32_t* flags = v->flags.as<uint32_t>();
   const uint32_t nblocks = (uint32_t)(v->words / kWordsPerBlock);
   if (num_points && p32)
     hipLaunchKernelGGL(k_vox_mark<float>, dim3(ceil_div(num_points, 256)), dim3(256), 0, stream,
-                       (const float*)points_fp16_dev, num_points, g, v->pkey.as<uint32_t>(), v->bitmap.as<uint32_t>());
+                       (const float*)points_fp16_dev, num_points, g, v->pkey.as<uint32_t>(), cells, flags);
   else if (num_points)
     hipLaunchKernelGGL(k_vox_mark<_Float16>, dim3(ceil_div(num_points, 256)), dim3(256), 0, stream,
-                       (const _Float16*)points_fp16_dev, num_points, g, v->pkey.as<uint32_t>(), v->bitmap.as<uint32_t>());
-  hipLaunchKernelGGL(k_bitmap_blocksum, dim3(nblocks), dim3(256), 0, stream, v->bitmap.as<uint32_t>(),
-                     v->blocksum.as<uint32_t>());
-  hipLaunchKernelGGL(k_scan_blocksums, dim3(1), dim3(1024), 0, stream, v->blocksum.as<uint32_t>(), nblocks, cnt,
-                     (uint32_t)p.max_voxels);
-  hipLaunchKernelGGL(k_bitmap_expand, dim3(nblocks), dim3(1024), 0, stream, v->bitmap.as<uint32_t>(),
-                     v->blocksum.as<uint32_t>(), Int3{{g.og[0], g.og[1], g.og[2]}}, (uint32_t)p.max_voxels,
-                     (int4*)v->idx.p, v->prefix.as<uint32_t>(), 0, (uint32_t*)nullptr);
+                       (const _Float16*)points_fp16_dev, num_points, g, v->pkey.as<uint32_t>(), cells, flags);
+  hipLaunchKernelGGL(k_vox_blocksum, dim3(nblocks), dim3(256), 0, stream, cells, flags, v->blocksum.as<uint32_t>());
+  hipLaunchKernelGGL(k_vox_rank, dim3(nblocks), dim3(256), 0, stream, cells, v->blocksum.as<uint32_t>(),
+                     Int3{{g.og[0], g.og[1], g.og[2]}}, (uint32_t)p.max_voxels, (int4*)v->idx.p, cnt, v->counts.as<uint32_t>());
   if (num_points) {
-    hipLaunchKernelGGL(k_vox_assign, dim3(ceil_div(num_points, 256)), dim3(256), 0, stream, v->pkey.as<uint32_t>(),
-                       num_points, v->bitmap.as<uint32_t>(), v->prefix.as<uint32_t>(), p.max_voxels,
-                       p.max_points_per_voxel, v->counts.as<uint32_t>(), v->mins.as<uint32_t>());
+    const dim3 pgrid(ceil_div(num_points, 256));
+    hipLaunchKernelGGL(k_vox_assign, pgrid, dim3(256), 0, stream, v->pkey.as<uint32_t>(), num_points, cells, p.max_voxels,
+                       p.max_points_per_voxel, tag_arrival, v->counts.as<uint32_t>(), v->mins.as<uint32_t>(), overflow, always);
+    for (int phase = 0; phase < 2; ++phase)
+      hipLaunchKernelGGL(k_vox_overflow, dim3(std::min(pgrid.x, 512u)), dim3(256), 0, stream, v->pkey.as<uint32_t>(),
+                         num_points, cells, p.max_voxels, p.max_points_per_voxel, tag_cascade, v->counts.as<uint32_t>(),
+                         v->mins.as<uint32_t>(), overflow, always, phase);
     const uint32_t bound = (uint32_t)std::min<uint64_t>((uint64_t)p.max_voxels, num_points);
+    const uint32_t threads = std::max(bound, num_points);
     if (p32)
-      hipLaunchKernelGGL(k_vox_mean<float>, dim3(ceil_div(bound * p.num_feature, 256)), dim3(256), 0, stream,
+      hipLaunchKernelGGL(k_vox_mean<float>, dim3(ceil_div(threads, 256)), dim3(256), 0, stream,
                          (const float*)points_fp16_dev, cnt, p.max_voxels, p.max_points_per_voxel, p.num_feature,
-                         v->counts.as<uint32_t>(), v->mins.as<uint32_t>(), (_Float16*)v->feats.p);
+                         v->counts.as<uint32_t>(), v->mins.as<uint32_t>(), (_Float16*)v->feats.p, v->pkey.as<uint32_t>(),
+                         num_points, cells, flags, overflow);
     else
-      hipLaunchKernelGGL(k_vox_mean<_Float16>, dim3(ceil_div(bound * p.num_feature, 256)), dim3(256), 0, stream,
+      hipLaunchKernelGGL(k_vox_mean<_Float16>, dim3(ceil_div(threads, 256)), dim3(256), 0, stream,
                          (const _Float16*)points_fp16_dev, cnt, p.max_voxels, p.max_points_per_voxel, p.num_feature,
-                         v->counts.as<uint32_t>(), v->mins.as<uint32_t>(), (_Float16*)v->feats.p);
+                         v->counts.as<uint32_t>(), v->mins.as<uint32_t>(), (_Float16*)v->feats.p, v->pkey.as<uint32_t>(),
+                         num_points, cells, flags, overflow);
   }
   SCN_HIP(hipGetLastError());
   if (debug_sync_enabled()) return debug_sync_check(stream, "scn_voxelizer_forward");

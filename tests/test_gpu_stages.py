@@ -649,11 +649,11 @@ def test_memset_kernel_any_alignment_and_inside_a_graph():
 
 
 # ----------------------------------------------------------------------------- voxelization
-def _voxelizer(max_voxels=160000, max_points=300000):
+def _voxelizer(max_voxels=160000, max_points=300000, per_voxel=10):
     p = capi.VoxelizationParam()
     p.min_range[:] = synth.MIN_RANGE; p.max_range[:] = synth.MAX_RANGE; p.voxel_size[:] = synth.VOXEL_SIZE
     p.grid_size[:] = synth.GRID_XYZ
-    p.num_feature, p.max_voxels, p.max_points_per_voxel, p.max_points = 5, max_voxels, 10, max_points
+    p.num_feature, p.max_voxels, p.max_points_per_voxel, p.max_points = 5, max_voxels, per_voxel, max_points
     h = capi.lib().scn_voxelizer_create(C.byref(p))
     assert h
     return h
@@ -724,6 +724,65 @@ def test_voxelization_of_fp32_points_bit_exact(order, nuscenes_frame):
         f2, i2, c2 = _run_voxelizer(h, nuscenes_frame[:50000], order, 160000)
         rf2, ri2, rc2 = O.voxelize(nuscenes_frame[:50000], synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, order=order)
         assert np.array_equal(i2, ri2) and np.array_equal(c2, rc2) and np.array_equal(f2.view(np.uint16), rf2.view(np.uint16))
+    finally:
+        L.scn_voxelizer_destroy(h)
+
+
+def test_voxelizer_state_survives_many_forwards(nuscenes_frame):
+    """The voxelizer cleans its working memory at the end of a forward instead of clearing it at the start, and tags
+    the per-voxel point slots with a call counter that is used up after 127 forwards: 600 forwards on one object,
+    alternating three frames (a ring-ordered real one, a synthetic one, a short one), checked against the oracle at
+    the first calls, around the wraps of the counter and at the end; then a frame that overflows max_voxels (cells
+    beyond the kept rows must be cleaned too) followed by an ordinary one."""
+    L = capi.lib()
+    frames = [nuscenes_frame[:120000], synth.lidar_frame(5, 90000), nuscenes_frame[200000:200700]]
+    want = [O.voxelize(f, synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, order="zyx") for f in frames]
+    devs = [to_dev(f) for f in frames]
+    h = _voxelizer()
+    try:
+        note("600 forwards on one voxelizer, three frames in turn")
+        for call in range(600):
+            k = call % 3
+            capi.check(L.scn_voxelizer_forward(h, ptr(devs[k]), frames[k].shape[0], capi.ORDER_ZYX, stream()))
+            if call < 6 or 120 <= call <= 135 or 250 <= call <= 262 or 376 <= call <= 388 or call >= 594:
+                nv = L.scn_voxelizer_num_voxels(h, stream())
+                f = copy_from_ptr(L.scn_voxelizer_features(h), (nv, 5), np.float16).cpu().numpy()
+                i = copy_from_ptr(L.scn_voxelizer_indices(h), (nv, 4), np.int32).cpu().numpy()
+                c = copy_from_ptr(L.scn_voxelizer_points_per_voxel(h), (nv,), np.int32).cpu().numpy()
+                rf, ri, rc = want[k]
+                assert np.array_equal(i, ri) and np.array_equal(c, rc), call
+                assert np.array_equal(f.view(np.uint16), rf.view(np.uint16)), call
+    finally:
+        L.scn_voxelizer_destroy(h)
+    note("a frame that overflows max_voxels, then an ordinary one on the same object")
+    h = _voxelizer(max_voxels=3000)
+    try:
+        f, i, c = _run_voxelizer(h, frames[0], "zyx", 3000)
+        rf, ri, rc = O.voxelize(frames[0], synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, max_voxels=3000, order="zyx")
+        assert f.shape[0] == 3000 and np.array_equal(i, ri) and np.array_equal(c, rc) and np.array_equal(f.view(np.uint16), rf.view(np.uint16))
+        f, i, c = _run_voxelizer(h, frames[2], "zyx", 3000)
+        rf, ri, rc = want[2]
+        assert np.array_equal(i, ri) and np.array_equal(c, rc) and np.array_equal(f.view(np.uint16), rf.view(np.uint16))
+    finally:
+        L.scn_voxelizer_destroy(h)
+
+
+@pytest.mark.parametrize("per_voxel", [1, 3, 16, 24])
+def test_voxelization_points_per_voxel_limits(per_voxel, nuscenes_frame):
+    """max_points_per_voxel of 1 and 3 (most voxels of a real sweep overflow: the lowest point indices must win whatever
+    the arrival order), 16 (the most that the mean kernel puts in order itself) and 24 (every voxel through the
+    cascade), two forwards each."""
+    note(f"voxelization with at most {per_voxel} points per voxel")
+    L = capi.lib()
+    h = _voxelizer(per_voxel=per_voxel)
+    try:
+        for pts in (nuscenes_frame[:150000], nuscenes_frame[100000:220000]):
+            f, i, c = _run_voxelizer(h, pts, "zyx", 160000)
+            rf, ri, rc = O.voxelize(pts, synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, max_points=per_voxel,
+                                    order="zyx")
+            assert np.array_equal(i, ri) and np.array_equal(c, rc)
+            assert np.array_equal(f.view(np.uint16), rf.view(np.uint16))
+            assert (rc > per_voxel).any()
     finally:
         L.scn_voxelizer_destroy(h)
 
