@@ -924,17 +924,18 @@ struct VoxGeom {
 //   flags     one word per block of 1024 words: some cell of the block is occupied; cleared the same way.  (Walking
 //             a second-level bitmap of the occupied words instead -- one thread per 32 words, 82 workgroups -- was
 //             measured at 16 + 46 us for the two rank passes against 5 + 17 us: few threads with dependent loads.)
-//   slots     [max_voxels][max_points] point indices tagged in the top 8 bits.  A forward uses two tags, 2e + 1 for
-//             the slots filled in arrival order and 2e for the cascade of the voxels that overflow, and e counts
-//             DOWN: every value of an earlier call (or phase) is larger than any value of the current one, so to the
-//             atomicMin cascade a stale slot is an empty one.  (A full clear every 127 calls, when the tags wrap.)
+//   slots     [max_voxels][max_points] point indices with a phase bit above them: 1 for the slots filled in arrival
+//             order, 0 for the cascade of the voxels that overflow, so that to the cascade (atomicMin) a slot of the
+//             arrival phase is an empty one.  Never cleared: a forward writes every slot that it reads or that its
+//             cascade can reach (the first min(count, max_points) of a voxel), so what earlier forwards left
+//             behind them is never looked at.  No state on the host either: a captured forward replays as it is.
 // Atomics that every XCD must see are the cost of this stage (they are served by the memory side, not by an XCD's L2),
 // so a point costs two: the occupancy bit, and its voxel's counter, whose old value is its slot.  A voxel that
 // receives more than max_points points needs the lowest indices among them, which arrival order does not give: those
 // voxels' points (none in most frames: the pass leaves at once when no counter overflowed) go through a cascade.
 // One forward = mark, block sums, rank, assign, overflow, mean.
 constexpr uint32_t kVoxTagShift = 24;     // point indices stay below 2^24
-constexpr uint32_t kVoxEpochs = 127;      // epochs 126 .. 0 (tags 253 .. 0); 255 is what a cleared slot holds
+constexpr uint32_t kVoxTagArrival = 1, kVoxTagCascade = 0;
 
 // Pass 1 over the point stream (PT: fp16 points, or the fp32 points of CUDA-CenterPoint's preprocessing,
 // src/preprocess_kernels.cu:70-98): cell key per point, occupancy bit, and the flag of the cell's block.
@@ -1114,10 +1115,14 @@ __global__ __launch_bounds__(256) void k_vox_overflow(const uint32_t* __restrict
     // (Loads at device scope: the atomics are carried out by the memory side, and an ordinary load could be served
     // from a copy that never sees them.  Read-modify-writes on one 64-byte line run one after the other, at about ten
     // per microsecond: without these reads the frame's fullest voxel alone sets the time of the pass.)
-    const uint32_t last = __hip_atomic_load(&slot[max_pts - 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if ((last >> kVoxTagShift) == tag && last < x) continue;
+    // (Not when every voxel takes this pass: a voxel with fewer points than slots then keeps, in the slots behind them,
+    // what an earlier forward's cascade left there, and those must not be read.)
     int j0 = 0;
-    for (; j0 < max_pts; ++j0) {
+    if (!always) {
+      const uint32_t last = __hip_atomic_load(&slot[max_pts - 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if ((last >> kVoxTagShift) == tag && last < x) continue;
+    }
+    for (; !always && j0 < max_pts; ++j0) {
       const uint32_t cur = __hip_atomic_load(&slot[j0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if ((cur >> kVoxTagShift) != tag || cur > x) break;
     }
@@ -1364,14 +1369,7 @@ int scn_voxelizer_forward_points(scn_voxelizer* v, const void* points_fp16_dev, 
   g.max_voxels = p.max_voxels;
   g.max_pts = p.max_points_per_voxel;
   v->last_order = order;
-  // (the working memory is clean: see the kernels.  The slots' tags count down; when they are used up the slots are cleared.)
-  if (v->epoch == 0) {
-    int rc = fill_u32(v->mins.p, 0xFFFFFFFFu, (size_t)p.max_voxels * p.max_points_per_voxel, stream);
-    if (rc) return rc;
-    v->epoch = kVoxEpochs;
-  }
-  const uint32_t epoch = --v->epoch;
-  const uint32_t tag_arrival = 2 * epoch + 1, tag_cascade = 2 * epoch;
+  const uint32_t tag_arrival = kVoxTagArrival, tag_cascade = kVoxTagCascade;   // (the working memory is clean: see the kernels)
   // (more slots or features than pass 4 puts in order in registers: every voxel goes through the cascade of pass 3b)
   const int always = (p.max_points_per_voxel > kVoxMaxSlots || p.num_feature > kVoxMaxFeatures) ? 1 : 0;
   uint32_t* cnt = v->counters.as<uint32_t>();

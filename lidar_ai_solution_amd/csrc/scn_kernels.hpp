@@ -227,7 +227,6 @@ struct scn_voxelizer {
   scn_voxelization_param p{};
   scn::DevBuf bitmap, blocksum, flags, pkey, mins, counts, feats, idx, counters;
   size_t words = 0;
-  uint32_t epoch = 127;            // the next forward's slot tags are 2 (epoch - 1) + 1 and 2 (epoch - 1): see k_vox_assign
   uint32_t* host_count = nullptr;  // pinned
   int last_order = SCN_ORDER_XYZ;
 };

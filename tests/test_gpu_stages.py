@@ -729,10 +729,10 @@ def test_voxelization_of_fp32_points_bit_exact(order, nuscenes_frame):
 
 
 def test_voxelizer_state_survives_many_forwards(nuscenes_frame):
-    """The voxelizer cleans its working memory at the end of a forward instead of clearing it at the start, and tags
-    the per-voxel point slots with a call counter that is used up after 127 forwards: 600 forwards on one object,
-    alternating three frames (a ring-ordered real one, a synthetic one, a short one), checked against the oracle at
-    the first calls, around the wraps of the counter and at the end; then a frame that overflows max_voxels (cells
+    """The voxelizer cleans its working memory at the end of a forward instead of clearing it at the start, and never
+    clears the per-voxel point slots at all (a forward writes every slot it reads): 600 forwards on one object,
+    alternating three frames (a ring-ordered real one with voxels that overflow, a synthetic one, a short one), checked
+    against the oracle at the first calls, at intervals and at the end; then a frame that overflows max_voxels (cells
     beyond the kept rows must be cleaned too) followed by an ordinary one."""
     L = capi.lib()
     frames = [nuscenes_frame[:120000], synth.lidar_frame(5, 90000), nuscenes_frame[200000:200700]]
