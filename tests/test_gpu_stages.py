@@ -787,6 +787,53 @@ def test_voxelization_points_per_voxel_limits(per_voxel, nuscenes_frame):
         L.scn_voxelizer_destroy(h)
 
 
+@pytest.mark.parametrize("per_voxel", [10, 24])
+def test_voxelizer_forward_replayed_from_a_graph(per_voxel, nuscenes_frame):
+    """A forward captured once into a HIP graph and replayed on other frames of the same point count (the graph fixes
+    the launch arguments, the point buffer's contents change): the voxelizer keeps no state on the host, so every
+    replay must equal the oracle -- with 10 slots per voxel (only the overflowing voxels go through the cascade) and
+    with 24 (every voxel does), direct forwards mixed in between."""
+    L = capi.lib()
+    n = 100000
+    frames = [nuscenes_frame[:n], nuscenes_frame[150000:150000 + n], synth.lidar_frame(8, n), nuscenes_frame[60000:60000 + n]]
+    want = [O.voxelize(f, synth.MIN_RANGE, synth.MAX_RANGE, synth.VOXEL_SIZE, synth.GRID_XYZ, max_points=per_voxel, order="zyx")
+            for f in frames]
+    note(f"voxelizer forward captured into a graph, {per_voxel} slots per voxel, replayed on four frames")
+    h = _voxelizer(per_voxel=per_voxel)
+    st = torch.cuda.Stream()
+    sp = C.c_void_p(st.cuda_stream)
+    buf = to_dev(frames[0]).clone()
+
+    def check(k, what):
+        nv = L.scn_voxelizer_num_voxels(h, sp)
+        f = copy_from_ptr(L.scn_voxelizer_features(h), (nv, 5), np.float16).cpu().numpy()
+        i = copy_from_ptr(L.scn_voxelizer_indices(h), (nv, 4), np.int32).cpu().numpy()
+        c = copy_from_ptr(L.scn_voxelizer_points_per_voxel(h), (nv,), np.int32).cpu().numpy()
+        rf, ri, rc = want[k]
+        assert np.array_equal(i, ri) and np.array_equal(c, rc), (what, k)
+        assert np.array_equal(f.view(np.uint16), rf.view(np.uint16)), (what, k)
+
+    try:
+        with torch.cuda.stream(st):
+            capi.check(L.scn_voxelizer_forward(h, ptr(buf), n, capi.ORDER_ZYX, sp))
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=st):
+            capi.check(L.scn_voxelizer_forward(h, ptr(buf), n, capi.ORDER_ZYX, sp))
+        torch.cuda.synchronize()
+        for rep, k in enumerate((1, 2, 0, 3, 3, 1)):
+            with torch.cuda.stream(st):
+                buf.copy_(to_dev(frames[k]))
+                if rep == 3:     # a direct forward on another frame between two replays
+                    other = to_dev(frames[2])
+                    capi.check(L.scn_voxelizer_forward(h, ptr(other), n, capi.ORDER_ZYX, sp))
+                g.replay()
+            torch.cuda.synchronize()
+            check(k, f"replay {rep}")
+    finally:
+        L.scn_voxelizer_destroy(h)
+
+
 def test_voxelization_truncates_at_max_voxels(nuscenes_frame):
     note("voxelization with max_voxels=5000")
     L = capi.lib()
