@@ -1090,7 +1090,9 @@ __global__ __launch_bounds__(256) void k_vox_assign(const uint32_t* __restrict__
 // the sensor holds a thousand points in a hundred runs, and read-modify-writes on one 64-byte line are carried out one
 // after the other by the memory side, about ten per microsecond: all candidates at once are over a thousand of them
 // (135 us on the reference's demo sweep), while after phase 0 the slots hold ten low indices and nearly every
-// other candidate leaves on the reads in front of the cascade.
+// other candidate leaves on the reads in front of the cascade (86 us for the two launches).  (A bound per voxel from
+// the indices that pass 3 happened to store -- the lowest max_pts cannot lie above the largest of any max_pts -- in
+// place of phase 0: 113 us; arrival order follows index order too loosely for it.)
 __global__ __launch_bounds__(256) void k_vox_overflow(const uint32_t* __restrict__ pkey, uint32_t n,
                                                       const uint2* __restrict__ cells, int max_voxels, int max_pts,
                                                       uint32_t tag, const uint32_t* __restrict__ counts, uint32_t* slots,
@@ -1207,9 +1209,9 @@ __global__ __launch_bounds__(256) void k_vox_mean(const PT* __restrict__ pts, co
   const uint32_t* slot = slots + (size_t)v * max_pts;
   const uint32_t pmask = (1u << kVoxTagShift) - 1u;
   _Float16* out = feats + (size_t)v * nf;
-  if (all > (uint32_t)max_pts || max_pts > kVoxMaxSlots || nf > kVoxMaxFeatures) {
-    // in order already (the cascade's result: see the host side for max_pts > 16), or more features than the
-    // registers below hold
+  if (max_pts > kVoxMaxSlots || nf > kVoxMaxFeatures) {
+    // more slots or features than the registers below hold: every voxel went through the cascade (see the host
+    // side), its slots are in order
     for (int f = 0; f < nf; ++f) {
       float s = 0.f;
       for (uint32_t j = 0; j < cnt; ++j) {
